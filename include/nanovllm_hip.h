@@ -571,8 +571,15 @@ int32_t nvh_residual_norm(const void* a, int64_t a_stride, const void* a_weight,
                           float branch_scale, float branch_eps, const void* c, int64_t c_stride, const float* c32, int64_t c32_stride,
                           float* x, int32_t norm_kind, const void* norm_weight, const void* norm_bias, float eps, void* h, int64_t h_stride,
                           int64_t rows, int64_t dim, int32_t act_f32, nvh_stream_t stream);
+/* The close of a sublayer in a stack that norms after the sum.  Per row:
+ *   v = alpha x + layer_scale (y + y32);   x <- v / sqrt(mean(v^2) + eps) * (weight_offset + norm_weight);   h <- x (type A)
+ * y (type A) and y32 (fp32) may be NULL (both NULL: the norm of alpha x alone); layer_scale [dim] (type A, NULL: 1); h may be
+ * NULL; write_x 0: x is read only.  All arithmetic in fp32. */
+int32_t nvh_residual_postnorm(const void* y, int64_t y_stride, const float* y32, int64_t y32_stride, const void* layer_scale, float alpha,
+                              float* x, int32_t write_x, const void* norm_weight, float weight_offset, float eps, void* h, int64_t h_stride,
+                              int64_t rows, int64_t dim, int32_t act_f32, nvh_stream_t stream);
 /* y[rows, inter] = act(x[:, :inter]) (* x[:, inter:2 inter] when gated), evaluated in fp32.  act 0: silu, 1: gelu (tanh form),
- * 2: squared relu. */
+ * 2: squared relu, 3: tanh. */
 int32_t nvh_act_mul(const void* x, int64_t row_stride, void* y, int64_t y_stride, int64_t rows, int64_t inter, int32_t act, int32_t gated,
                     int32_t act_f32, nvh_stream_t stream);
 /* out fp32 [rows, vocab] = scale * logits, softcapped when cap > 0. */
@@ -587,21 +594,31 @@ int32_t nvh_logits_scale(const void* logits, int64_t row_stride, float* out, int
  * nvh_scan_segmentable holds; ignored otherwise): a sequence that brings at least segment_min_tokens tokens is cut into that
  * many segments walked side by side and joined in a second launch; ws_states fp32 [batch, H, segments, dv, dk] and ws_decays
  * fp32 [batch, H, segments, dk] are scratch.  Results then differ from the unsegmented form within rounding.
+ * read_first: a token is read out before it is written and decayed, o = (S + diag(u) (c k) v^T)^T q + d v, then
+ * S <- diag(w) S + (c k) v^T, with the bonus u fp32 [H, dk] (NULL: 0) for the token itself (the RWKV time mix).
  * nvh_hgrn2_prep: q = silu(q), w = f = lower + (1 - lower) sigmoid(f + f_bias), k = 1 - f, v.
- * nvh_gla_prep: q * q_scale, k, v, w = sigmoid(decay_logits)^(1 / tau) (decay_logits fp32).
+ * nvh_gla_prep: q * q_scale, k, v, w = sigmoid(decay_logits)^(1 / tau) (decay_logits fp32; decay_kind 0), or
+ * w = exp(-exp(decay_logits)) (decay_kind 1).
+ * nvh_token_shift_mix: out[s, t, :] (type A, [num_mixes, T, dim]) = h_t + (h_(t-1) - h_t) mu[s, :], h_(t-1) of a step's
+ * first token taken from state fp32 [slots, dim] (zeros at a sequence's start); nvh_conv_state_update with two taps
+ * then leaves every sequence's last h in its slot.
+ * nvh_rotary_qkv_prep: fp32 q, k [T, H dim] and v [T, H vdim] from projection columns, rotary positions on the first
+ * rot_dims dimensions of every q / k head (angle = position freq[pair], cos and sin times mag; interleaved pairs
+ * (2i, 2i + 1) or halves (i, i + rot_dims / 2)), then q * q_scale and k * k_scale.
  * nvh_ssd_conv_prep: the causal convolution (weights [C, taps], last tap on the current token; bias NULL: none) over the
  * C = inner + 2 gn channels x | B | C of every token, continued from the sequence's carried inputs conv_state
  * [slots, taps - 1, C] (zeros at a sequence's start), then silu -> out_x [T, inner], out_b, out_c [T, gn];
  * out_dt = softplus(dt + dt_bias) and out_decay = exp(-exp(a_log) out_dt), both [T, H].
  * nvh_conv_state_update (after nvh_ssd_conv_prep of the same step): the last taps - 1 inputs of every sequence -> its slot.
  * nvh_group_rmsnorm_gate: y (type A) = unit over groups of group_size columns of o (o * gate first when gate_first),
- * times weight ([group_size] shared, or [groups group_size] when weight_full), times gate afterwards otherwise;
+ * times weight ([group_size] shared, or [groups group_size] when weight_full; NULL: none), times gate afterwards otherwise;
  * gate_act 0: no gate, 1: sigmoid(gate), 2: silu(gate). */
 int32_t nvh_gated_linear_scan(const float* q, int64_t q_stride, const float* k, int64_t k_stride, int64_t qk_groups, const float* w,
                               int64_t w_stride, int32_t w_scalar, const float* kscale, int64_t kscale_stride, const float* v,
                               int64_t v_stride, const float* skip, float* state, const int32_t* slots, const int32_t* cu_seqlens_q,
                               const int32_t* context_lens, float* out, int64_t batch, int64_t heads, int64_t dk, int64_t dv,
-                              int64_t segments, int64_t segment_min_tokens, float* ws_states, float* ws_decays, nvh_stream_t stream);
+                              int64_t segments, int64_t segment_min_tokens, float* ws_states, float* ws_decays, int32_t read_first,
+                              const float* bonus, nvh_stream_t stream);
 /* Whether key size dk has the segmented form of the scan. */
 int32_t nvh_scan_segmentable(int64_t dk);
 int32_t nvh_hgrn2_prep(const void* q, int64_t q_stride, const void* f, int64_t f_stride, const void* v, int64_t v_stride,
@@ -609,7 +626,15 @@ int32_t nvh_hgrn2_prep(const void* q, int64_t q_stride, const void* f, int64_t f
                        int64_t num_tokens, int64_t n_k, int64_t n_v, int32_t act_f32, nvh_stream_t stream);
 int32_t nvh_gla_prep(const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v, int64_t v_stride,
                      const float* decay_logits, int64_t z_stride, float q_scale, float tau, float* out_q, float* out_k,
-                     float* out_w, float* out_v, int64_t num_tokens, int64_t n_k, int64_t n_v, int32_t act_f32, nvh_stream_t stream);
+                     float* out_w, float* out_v, int64_t num_tokens, int64_t n_k, int64_t n_v, int32_t decay_kind, int32_t act_f32,
+                     nvh_stream_t stream);
+int32_t nvh_token_shift_mix(const void* h, int64_t h_stride, const float* state, const int32_t* slots, const int32_t* cu_seqlens_q,
+                            const int32_t* context_lens, int64_t batch, const void* mu, void* out, int64_t num_tokens, int64_t num_mixes,
+                            int64_t dim, int32_t act_f32, nvh_stream_t stream);
+int32_t nvh_rotary_qkv_prep(const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v, int64_t v_stride,
+                            const int64_t* positions, const float* freq, float mag, int64_t rot_dims, int32_t interleaved, float q_scale,
+                            float k_scale, float* out_q, float* out_k, float* out_v, int64_t num_tokens, int64_t heads, int64_t dim,
+                            int64_t vdim, int32_t act_f32, nvh_stream_t stream);
 int32_t nvh_ssd_conv_prep(const void* xbc, int64_t xbc_stride, const void* dt, int64_t dt_stride, const void* conv_w, const void* conv_b,
                           const void* dt_bias, const void* a_log, float* conv_state, const int32_t* slots, const int32_t* cu_seqlens_q,
                           const int32_t* context_lens, int64_t batch, int64_t num_tokens, int64_t taps, int64_t heads, int64_t inner,
@@ -626,7 +651,8 @@ int32_t nvh_group_rmsnorm_gate(const float* o, const void* weight, int32_t weigh
  * src_token[pos] = the pair's token, pos_of_pair[pair] = its position, and tiles of up to 64 positions of one expert
  * (tile_expert, tile_row0, tile_rows; unused tiles have 0 rows); max_tiles >= nvh_moe_max_tiles(T top, E).
  * nvh_gemm_grouped_any_nt: y[pos] = x[gather ? gather[pos] : pos] w[expert]^T over the tiles, w [E, N, K]; types as
- * nvh_gemm_any_nt.  nvh_moe_combine: out fp32 [T, dim] = sum_r weights[t, r] y[pos_of_pair[t, r]] (+ shared[t], type A). */
+ * nvh_gemm_any_nt.  nvh_moe_combine: out fp32 [T, dim] = sum_r weights[t, r] y[pos_of_pair[t, r]] (+ shared[t], type A,
+ * times sigmoid(shared_gate[t shared_gate_stride]) when a gate logit per token is given). */
 int32_t nvh_moe_route(const float* logits, int64_t row_stride, int32_t* ids, float* weights, int64_t num_tokens, int64_t experts,
                       int64_t top, nvh_stream_t stream);
 /* nvh_moe_route with the router's product inside: logits = x w^T + bias (x [T, K], w [E, K], bias [E] or NULL, type A;
@@ -641,7 +667,33 @@ int32_t nvh_gemm_grouped_any_nt(const void* x, int64_t x_row_stride, const int32
                                 const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* tile_rows, int64_t max_tiles,
                                 int64_t N, int64_t K, int32_t in_f32, int32_t out_f32, nvh_stream_t stream);
 int32_t nvh_moe_combine(const void* y, int64_t y_row_stride, const int32_t* pos_of_pair, const float* weights, const void* shared,
-                        int64_t shared_stride, float* out, int64_t num_tokens, int64_t dim, int64_t top, int32_t act_f32, nvh_stream_t stream);
+                        int64_t shared_stride, const float* shared_gate, int64_t shared_gate_stride, float* out, int64_t num_tokens, int64_t dim,
+                        int64_t top, int32_t act_f32, nvh_stream_t stream);
+/* Routing by scores: s = softmax(x w^T) over all experts (fp32); choice scores s + correction ([E], type A, or NULL);
+ * `groups` equal groups of neighbouring experts, a group's score its largest choice score, only the `keep` best groups
+ * eligible (groups 1: no restriction); the `top` best eligible experts (ties: lower id) -> ids, weights = their s times
+ * scale (not renormalised).  aux [num_aux, K] (type A, or NULL): further rows over the same input, their fp32 products
+ * -> aux_out [T, num_aux].  scores_out fp32 [T, E] or NULL. */
+int32_t nvh_moe_route_scored(const void* x, int64_t x_row_stride, const void* w, const void* correction, const void* aux, float* aux_out,
+                             int64_t num_aux, int32_t* ids, float* weights, float* scores_out, int64_t num_tokens, int64_t experts, int64_t K,
+                             int64_t top, int64_t groups, int64_t keep, float scale, int32_t act_f32, nvh_stream_t stream);
+
+/* Attention through a low-rank latent (csrc/latent_attention.hip).  nvh_latent_prep, per token over the projection row
+ * [dq (q_rank) | dkv (kv_rank + rot_dim, only with own_kv) | gate (heads, only with gate_out)]: cq_out (type A) = RMS norm
+ * of dq times q_norm_weight; with own_kv the RMS-normed latent times kv_norm_weight and the rotated shared key part go to
+ * the token's slot of k_cache [pages, page, 1, kv_rank + rot_dim], the latent once more to v_cache [pages, 1, kv_rank, page];
+ * gate_out fp32 [T, heads] = sigmoid.  nvh_latent_q_rotary: out[t, h, out_offset + d] = rotary of q[t, h, dim + d], d < rot_dim
+ * (q rows [heads, dim + rot_dim], out rows [heads, out_head_size]).  nvh_gemm_heads_nt: y[m, h, :N] = x[m, h, :K] w[h]^T,
+ * w [heads, N, K], head h at x + h x_head_stride / y + h y_head_stride within a row; y of type A. */
+int32_t nvh_latent_prep(const void* proj, int64_t proj_row_stride, int64_t q_rank, int64_t kv_rank, int64_t rot_dim, int64_t heads, int32_t own_kv,
+                        const void* q_norm_weight, const void* kv_norm_weight, float eps, const int64_t* positions, const float* freq, float mag,
+                        int32_t interleaved, void* cq_out, float* gate_out, void* k_cache, void* v_cache, const int32_t* slot_mapping,
+                        int64_t page, int64_t num_tokens, int32_t act_f32, nvh_stream_t stream);
+int32_t nvh_latent_q_rotary(const void* q, int64_t q_row_stride, const int64_t* positions, const float* freq, float mag, int32_t interleaved,
+                            void* out, int64_t out_row_stride, int64_t num_tokens, int64_t heads, int64_t dim, int64_t rot_dim,
+                            int64_t out_head_size, int64_t out_offset, int32_t act_f32, nvh_stream_t stream);
+int32_t nvh_gemm_heads_nt(const void* x, int64_t x_row_stride, int64_t x_head_stride, const void* w, void* y, int64_t y_row_stride,
+                          int64_t y_head_stride, int64_t M, int64_t heads, int64_t N, int64_t K, int32_t act_f32, nvh_stream_t stream);
 
 #ifdef __cplusplus
 }

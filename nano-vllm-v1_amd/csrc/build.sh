@@ -8,7 +8,7 @@ HIPCC="${HIPCC:-/opt/rocm/bin/hipcc}"
 # (packed fp32 arithmetic is switched off: the compiler then never forms v_pk_*_f32 from scalar float code)
 FLAGS="--offload-arch=gfx950 -O3 -std=c++17 -fPIC -ffp-contract=off -Wall -Wno-unused-function -Xclang -target-feature -Xclang -packed-fp32-ops"
 pids=()
-for f in api elementwise attention_decode attention_prefill gemm sampler comm model_forward stream_f32 attention_any delta_rule linear_recurrence moe; do
+for f in api elementwise attention_decode attention_prefill gemm sampler comm model_forward stream_f32 attention_any delta_rule linear_recurrence moe latent_attention; do
     if [ ! -f "$here/.obj/$f.o" ] || [ "$here/$f.hip" -nt "$here/.obj/$f.o" ] || [ "$here/common.h" -nt "$here/.obj/$f.o" ] || [ "$here/gemm_any.h" -nt "$here/.obj/$f.o" ] || [ "$here/../../include/nanovllm_hip.h" -nt "$here/.obj/$f.o" ]; then
         $HIPCC $FLAGS -c "$here/$f.hip" -o "$here/.obj/$f.o" &
         pids+=($!)

@@ -170,6 +170,44 @@ __device__ __forceinline__ void nvh_load8(const A* p, int64_t off, int valid, bo
     }
 }
 
+// ---- rotary positions ---------------------------------------------------------------------------
+// sin and cos of an fp32 angle through the hardware's sin(2 pi x) / cos(2 pi x): the turn count is reduced in float64 (an
+// angle of thousands of radians keeps its fp32 value exactly), the functions themselves are good to about 1e-6 absolute.
+// For the bf16 path; the library's sinf / cosf (used where everything is fp32) cost a few hundred instructions at such angles.
+__device__ __forceinline__ void sincos_turns(float ang, float& sn, float& cs) {
+    double rev = (double)ang * 0.15915494309189535;
+    rev -= floor(rev);
+    const float rf = (float)rev;
+    sn = __builtin_amdgcn_sinf(rf);
+    cs = __builtin_amdgcn_cosf(rf);
+}
+
+// The rotation's sine and cosine for activations of type A: the library functions where everything is fp32, the hardware
+// path where the result is rounded to bf16 anyway.
+template <typename A>
+__device__ __forceinline__ void rot_sincos(float ang, float& sn, float& cs) {
+    if constexpr (sizeof(A) == 4) {
+        sn = sinf(ang);
+        cs = cosf(ang);
+    } else {
+        sincos_turns(ang, sn, cs);
+    }
+}
+
+// Index of the rotation partner of element i among `n` rotated dimensions, and the pair number.
+__device__ __forceinline__ void pair_of(int i, int n, int interleaved, int& partner, int& pair, bool& first) {
+    if (interleaved) {
+        partner = i ^ 1;
+        pair = i >> 1;
+        first = (i & 1) == 0;
+    } else {
+        const int half = n >> 1;
+        first = i < half;
+        partner = first ? i + half : i - half;
+        pair = first ? i : i - half;
+    }
+}
+
 // ---- sampling pieces shared by the sampler kernels and the LM-head GEMM epilogue ------------------
 struct ValIdx {
     float v;

@@ -69,6 +69,7 @@ struct GlaPrepArgs {
     float q_scale, inv_tau;
     float *oq, *ok, *ow, *ov;
     int64_t n_k, n_v;
+    int decay_kind;            // 0: sigmoid(z)^(1/tau); 1: exp(-exp(z))
 };
 
 template <typename A>
@@ -77,9 +78,88 @@ __global__ __launch_bounds__(256) void gla_prep_kernel(GlaPrepArgs p) {
     for (int64_t i = threadIdx.x; i < p.n_k; i += 256) {
         p.oq[t * p.n_k + i] = ldf((const A*)p.q, t * p.q_stride + i) * p.q_scale;
         p.ok[t * p.n_k + i] = ldf((const A*)p.k, t * p.k_stride + i);
-        p.ow[t * p.n_k + i] = expf(logsigmoid_(p.z[t * p.z_stride + i]) * p.inv_tau);      // sigmoid(z)^(1/tau)
+        const float z = p.z[t * p.z_stride + i];
+        p.ow[t * p.n_k + i] = p.decay_kind == 1 ? expf(-expf(z)) : expf(logsigmoid_(z) * p.inv_tau);      // sigmoid(z)^(1/tau)
     }
     for (int64_t i = threadIdx.x; i < p.n_v; i += 256) p.ov[t * p.n_v + i] = ldf((const A*)p.v, t * p.v_stride + i);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Token shift: every token's input h is blended with the input of the token before it, with a weight vector per consumer,
+//   out[s, t, :] = h_t + (h_(t-1) - h_t) mu[s, :],   s = 0 .. n - 1,
+// where h_(t-1) of a step's first token is the input the sequence's slot carries (zeros at a sequence's start).  The
+// slot is brought up to date by nvh_conv_state_update afterwards (the carried input of a convolution with two taps).
+struct ShiftArgs {
+    const void* h;             // [T, D]
+    int64_t h_stride;
+    const float* state;        // [slots, D]
+    const int32_t *slots, *cu_seqlens_q, *context_lens;
+    int batch;
+    const void* mu;            // [n, D]
+    void* out;                 // [n, T, D]
+    int64_t tokens;
+    int n, D;
+};
+
+template <typename A>
+__global__ __launch_bounds__(256) void token_shift_mix_kernel(ShiftArgs p) {
+    const int64_t t = blockIdx.x;
+    const int seq = seq_of_token(p.cu_seqlens_q, p.batch, t);
+    const int lo = p.cu_seqlens_q ? p.cu_seqlens_q[seq] : seq, hi = p.cu_seqlens_q ? p.cu_seqlens_q[seq + 1] : seq + 1;
+    const int slot = p.slots[seq];
+    const bool first = (int)t == lo;
+    const bool carried = slot >= 0 && p.context_lens[seq] != hi - lo;
+    const A* cur = (const A*)p.h + t * p.h_stride;
+    const A* prev = first ? nullptr : cur - p.h_stride;
+    const float* st = first && carried ? p.state + (int64_t)slot * p.D : nullptr;
+    for (int i = threadIdx.x; i < p.D; i += 256) {
+        const float c = (float)cur[i];
+        const float b = prev ? (float)prev[i] : (st ? st[i] : 0.f);
+        const float d = b - c;
+        for (int s = 0; s < p.n; ++s)
+            ((A*)p.out)[((int64_t)s * p.tokens + t) * p.D + i] = (A)(c + d * (float)((const A*)p.mu)[(int64_t)s * p.D + i]);
+    }
+}
+
+// q, k, v projection columns -> the scan's fp32 operands with rotary positions on the first rot_dims dimensions of every q
+// and k head (angle = position * freq[pair], cos and sin times `mag`), q and k scaled AFTER the rotation.
+struct RotPrepArgs {
+    const void *q, *k, *v;
+    int64_t q_stride, k_stride, v_stride;
+    const int64_t* positions;
+    const float* freq;         // [rot_dims / 2] or null (rot_dims 0)
+    float mag, q_scale, k_scale;
+    int rot_dims, interleaved, H, dim, vdim;
+    float *oq, *ok, *ov;
+};
+
+template <typename A>
+__global__ __launch_bounds__(256) void rotary_qkv_prep_kernel(RotPrepArgs a) {
+    const int64_t t = blockIdx.x;
+    const float pos = (float)a.positions[t];
+    const int nk = a.H * a.dim, nv = a.H * a.vdim;
+    for (int which = 0; which < 2; ++which) {
+        const A* src = (const A*)(which ? a.k : a.q) + t * (which ? a.k_stride : a.q_stride);
+        float* dst = (which ? a.ok : a.oq) + t * nk;
+        const float scale = which ? a.k_scale : a.q_scale;
+        for (int i = threadIdx.x; i < nk; i += 256) {
+            const int d = i % a.dim;
+            float v = (float)src[i];
+            if (d < a.rot_dims) {
+                int partner, pair;
+                bool first;
+                pair_of(d, a.rot_dims, a.interleaved, partner, pair, first);
+                const float o = (float)src[i - d + partner];
+                float sn, cs;
+                rot_sincos<A>(pos * a.freq[pair], sn, cs);
+                const float c = cs * a.mag, s = sn * a.mag;
+                v = first ? v * c - o * s : v * c + o * s;
+            }
+            dst[i] = v * scale;
+        }
+    }
+    const A* vr = (const A*)a.v + t * a.v_stride;
+    for (int i = threadIdx.x; i < nv; i += 256) a.ov[t * nv + i] = (float)vr[i];
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -229,6 +309,7 @@ struct ScanArgs {
     int H, dk, dv;
     int nseg, seg_min;         // segments per long portion (1: none) and the fewest tokens that are cut
     float *ws_l, *ws_d;        // records of the segments: end states [batch, H, nseg, dv, dk] and decay products [batch, H, nseg, dk]
+    const float* bonus;        // PRE only: [H, dk] or null (0)
 };
 
 // Lanes per state column (SUBS), rows held per lane (DKQ), EXACT: dk == DKQ * SUBS (no loop carries a run-time bound; rows
@@ -243,7 +324,11 @@ struct ScanArgs {
 // folded from the records, adds (P_t q_t)^T S_j to every output of the segment (P_t: the product of the segment's decays
 // up to t), and the last segment leaves the sequence's state.  Products only, no division: a decay that underflows is a
 // zero.  A sequence with fewer than `seg_min` tokens in the step is one segment (MODE 1 then does all of it).
-template <int DKQ, int SUBS, bool EXACT, int MODE>
+//
+// PRE: the token is read out BEFORE it is written and decayed, with a bonus u per key channel for the token itself,
+//   o = (S + diag(u) (c k) v^T)^T q (+ d v),   S <- diag(w) S + (c k) v^T,
+// the form of the RWKV time mix.  The joining launch then weighs a segment's start state by the decays BEFORE the token.
+template <int DKQ, int SUBS, bool EXACT, int MODE, bool PRE>
 __global__ __launch_bounds__(256) void gated_linear_scan_kernel(ScanArgs p) {
     constexpr int COLS = 256 / SUBS;
     constexpr int CH = (3 * DKQ * SUBS + COLS + 4 + 255) / 256;     // loads per lane and token
@@ -269,7 +354,11 @@ __global__ __launch_bounds__(256) void gated_linear_scan_kernel(ScanArgs p) {
     constexpr bool VEC4 = EXACT && DKQ % 4 == 0;
     auto row_of = [&](int ii) { return VEC4 ? 4 * SUBS * (ii >> 2) + 4 * sub + (ii & 3) : SUBS * ii + sub; };
     auto row_ok = [&](int ii) { return EXACT || row_of(ii) < dk; };
-    float S[DKQ], P[DKQ];
+    float S[DKQ], P[DKQ], U[PRE ? DKQ : 1];
+    if constexpr (PRE) {
+#pragma unroll
+        for (int ii = 0; ii < DKQ; ++ii) U[ii] = (p.bonus && row_ok(ii)) ? p.bonus[(int64_t)head * dk + row_of(ii)] : 0.f;
+    }
 #pragma unroll
     for (int ii = 0; ii < DKQ; ++ii) {
         P[ii] = 1.f;
@@ -365,8 +454,18 @@ __global__ __launch_bounds__(256) void gated_linear_scan_kernel(ScanArgs p) {
             for (int ii = 0; ii < DKQ; ++ii)
                 if (EXACT || ii < dkq) {
                     if constexpr (MODE == 2) {
-                        P[ii] *= xw[ii];
-                        o = __builtin_fmaf(P[ii] * xq[ii], S[ii], o);
+                        if constexpr (PRE) {
+                            o = __builtin_fmaf(P[ii] * xq[ii], S[ii], o);
+                            P[ii] *= xw[ii];
+                        } else {
+                            P[ii] *= xw[ii];
+                            o = __builtin_fmaf(P[ii] * xq[ii], S[ii], o);
+                        }
+                    } else if constexpr (PRE) {
+                        const float kv = xk[ii] * sv;
+                        o = __builtin_fmaf(__builtin_fmaf(U[ii], kv, S[ii]), xq[ii], o);
+                        S[ii] = __builtin_fmaf(xw[ii], S[ii], kv);
+                        if constexpr (MODE == 1) P[ii] *= xw[ii];
                     } else {
                         const float sn = __builtin_fmaf(xw[ii], S[ii], xk[ii] * sv);
                         S[ii] = sn;
@@ -458,7 +557,7 @@ __global__ __launch_bounds__(256) void group_rmsnorm_gate_kernel(const float* __
     const float inv = 1.0f / sqrtf(ss / (float)gs + eps);
     for (int i = lane; i < gs; i += 64) {
         float v = pre ? orow[i] * gate_of(i) : orow[i];
-        v = v * inv * ldf(weight, w_full ? (int64_t)g * gs + i : i);
+        v = v * inv * (weight ? ldf(weight, w_full ? (int64_t)g * gs + i : i) : 1.0f);
         if (post) v *= gate_of(i);
         y[t * y_stride + (int64_t)g * gs + i] = (A)v;
     }
@@ -497,15 +596,15 @@ __global__ __launch_bounds__(256) void group_rmsnorm_gate_block_kernel(const flo
     for (int j = 0; j < PER; ++j) {
         const int i = threadIdx.x + 256 * j;
         if (i < gs) {
-            float r = v[j] * inv * ldf(weight, w_full ? (int64_t)g * gs + i : i);
+            float r = v[j] * inv * (weight ? ldf(weight, w_full ? (int64_t)g * gs + i : i) : 1.0f);
             if (post) r *= gv[j];
             y[t * y_stride + (int64_t)g * gs + i] = (A)r;
         }
     }
 }
 
-template <int DKQ, int SUBS, bool EXACT>
-void launch_scan_as(const ScanArgs& p, int64_t batch, hipStream_t st) {
+template <int DKQ, int SUBS, bool EXACT, bool PRE>
+void launch_scan_pre(const ScanArgs& p, int64_t batch, hipStream_t st) {
     constexpr int COLS = 256 / SUBS;
     constexpr int CH = (3 * DKQ * SUBS + COLS + 4 + 255) / 256;
     constexpr int TOK = (32 / CH) < 2 ? 2 : (32 / CH);
@@ -514,12 +613,18 @@ void launch_scan_as(const ScanArgs& p, int64_t batch, hipStream_t st) {
     if constexpr (EXACT) {
         if (p.nseg > 1) {
             const dim3 grid((unsigned)batch, (unsigned)p.H, colblocks * (unsigned)p.nseg);
-            gated_linear_scan_kernel<DKQ, SUBS, EXACT, 1><<<grid, 256, lds, st>>>(p);
-            gated_linear_scan_kernel<DKQ, SUBS, EXACT, 2><<<grid, 256, lds, st>>>(p);
+            gated_linear_scan_kernel<DKQ, SUBS, EXACT, 1, PRE><<<grid, 256, lds, st>>>(p);
+            gated_linear_scan_kernel<DKQ, SUBS, EXACT, 2, PRE><<<grid, 256, lds, st>>>(p);
             return;
         }
     }
-    gated_linear_scan_kernel<DKQ, SUBS, EXACT, 0><<<dim3((unsigned)batch, (unsigned)p.H, colblocks), 256, lds, st>>>(p);
+    gated_linear_scan_kernel<DKQ, SUBS, EXACT, 0, PRE><<<dim3((unsigned)batch, (unsigned)p.H, colblocks), 256, lds, st>>>(p);
+}
+
+template <int DKQ, int SUBS, bool EXACT>
+void launch_scan_as(const ScanArgs& p, int64_t batch, int read_first, hipStream_t st) {
+    if (read_first) launch_scan_pre<DKQ, SUBS, EXACT, true>(p, batch, st);
+    else launch_scan_pre<DKQ, SUBS, EXACT, false>(p, batch, st);
 }
 
 }  // namespace
@@ -540,15 +645,48 @@ extern "C" int32_t nvh_hgrn2_prep(const void* q, int64_t q_stride, const void* f
 
 extern "C" int32_t nvh_gla_prep(const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v, int64_t v_stride,
                                 const float* decay_logits, int64_t z_stride, float q_scale, float tau, float* out_q, float* out_k,
-                                float* out_w, float* out_v, int64_t num_tokens, int64_t n_k, int64_t n_v, int32_t act_f32, nvh_stream_t stream) {
+                                float* out_w, float* out_v, int64_t num_tokens, int64_t n_k, int64_t n_v, int32_t decay_kind, int32_t act_f32,
+                                nvh_stream_t stream) {
     NVH_REQUIRE(q && k && v && decay_logits && out_q && out_k && out_w && out_v, NVH_EINVAL, "nvh_gla_prep: null pointer");
-    NVH_REQUIRE(num_tokens >= 0 && n_k > 0 && n_v > 0 && tau > 0.f, NVH_EINVAL, "nvh_gla_prep: bad sizes");
+    NVH_REQUIRE(num_tokens >= 0 && n_k > 0 && n_v > 0 && tau > 0.f && (decay_kind == 0 || decay_kind == 1), NVH_EINVAL, "nvh_gla_prep: bad sizes");
     if (num_tokens == 0) return NVH_OK;
-    const GlaPrepArgs p{q, k, v, q_stride, k_stride, v_stride, decay_logits, z_stride, q_scale, 1.0f / tau, out_q, out_k, out_w, out_v, n_k, n_v};
+    const GlaPrepArgs p{q, k, v, q_stride, k_stride, v_stride, decay_logits, z_stride, q_scale, 1.0f / tau, out_q, out_k, out_w, out_v, n_k, n_v, decay_kind};
     hipStream_t st = (hipStream_t)stream;
     if (act_f32) gla_prep_kernel<float><<<dim3((unsigned)num_tokens), 256, 0, st>>>(p);
     else gla_prep_kernel<bf16><<<dim3((unsigned)num_tokens), 256, 0, st>>>(p);
     NVH_CHECK_LAUNCH("nvh_gla_prep");
+    return NVH_OK;
+}
+
+extern "C" int32_t nvh_token_shift_mix(const void* h, int64_t h_stride, const float* state, const int32_t* slots, const int32_t* cu_seqlens_q,
+                                       const int32_t* context_lens, int64_t batch, const void* mu, void* out, int64_t num_tokens, int64_t num_mixes,
+                                       int64_t dim, int32_t act_f32, nvh_stream_t stream) {
+    NVH_REQUIRE(h && state && slots && context_lens && mu && out, NVH_EINVAL, "nvh_token_shift_mix: null pointer");
+    NVH_REQUIRE(batch >= 0 && num_tokens >= 0 && num_mixes > 0 && dim > 0 && h_stride >= dim && (cu_seqlens_q || num_tokens == batch), NVH_EINVAL,
+                "nvh_token_shift_mix: bad sizes");
+    if (num_tokens == 0 || batch == 0) return NVH_OK;
+    const ShiftArgs p{h, h_stride, state, slots, cu_seqlens_q, context_lens, (int)batch, mu, out, num_tokens, (int)num_mixes, (int)dim};
+    hipStream_t st = (hipStream_t)stream;
+    if (act_f32) token_shift_mix_kernel<float><<<dim3((unsigned)num_tokens), 256, 0, st>>>(p);
+    else token_shift_mix_kernel<bf16><<<dim3((unsigned)num_tokens), 256, 0, st>>>(p);
+    NVH_CHECK_LAUNCH("nvh_token_shift_mix");
+    return NVH_OK;
+}
+
+extern "C" int32_t nvh_rotary_qkv_prep(const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v, int64_t v_stride,
+                                       const int64_t* positions, const float* freq, float mag, int64_t rot_dims, int32_t interleaved, float q_scale,
+                                       float k_scale, float* out_q, float* out_k, float* out_v, int64_t num_tokens, int64_t heads, int64_t dim,
+                                       int64_t vdim, int32_t act_f32, nvh_stream_t stream) {
+    NVH_REQUIRE(q && k && v && positions && out_q && out_k && out_v, NVH_EINVAL, "nvh_rotary_qkv_prep: null pointer");
+    NVH_REQUIRE(num_tokens >= 0 && heads > 0 && dim > 0 && vdim > 0 && rot_dims >= 0 && rot_dims <= dim && rot_dims % 2 == 0 && (rot_dims == 0 || freq),
+                NVH_EINVAL, "nvh_rotary_qkv_prep: bad sizes");
+    if (num_tokens == 0) return NVH_OK;
+    const RotPrepArgs a{q, k, v, q_stride, k_stride, v_stride, positions, freq, mag, q_scale, k_scale, (int)rot_dims, interleaved, (int)heads, (int)dim,
+                        (int)vdim, out_q, out_k, out_v};
+    hipStream_t st = (hipStream_t)stream;
+    if (act_f32) rotary_qkv_prep_kernel<float><<<dim3((unsigned)num_tokens), 256, 0, st>>>(a);
+    else rotary_qkv_prep_kernel<bf16><<<dim3((unsigned)num_tokens), 256, 0, st>>>(a);
+    NVH_CHECK_LAUNCH("nvh_rotary_qkv_prep");
     return NVH_OK;
 }
 
@@ -623,13 +761,15 @@ extern "C" int32_t nvh_gated_linear_scan(const float* q, int64_t q_stride, const
                                          int64_t w_stride, int32_t w_scalar, const float* kscale, int64_t kscale_stride, const float* v,
                                          int64_t v_stride, const float* skip, float* state, const int32_t* slots, const int32_t* cu_seqlens_q,
                                          const int32_t* context_lens, float* out, int64_t batch, int64_t heads, int64_t dk, int64_t dv,
-                                         int64_t segments, int64_t segment_min_tokens, float* ws_states, float* ws_decays, nvh_stream_t stream) {
+                                         int64_t segments, int64_t segment_min_tokens, float* ws_states, float* ws_decays, int32_t read_first,
+                                         const float* bonus, nvh_stream_t stream) {
     NVH_REQUIRE(q && k && w && v && state && slots && context_lens && out, NVH_EINVAL, "nvh_gated_linear_scan: null pointer");
     NVH_REQUIRE(batch >= 0 && heads > 0 && dk > 0 && dv > 0 && qk_groups > 0 && heads % qk_groups == 0, NVH_EINVAL, "nvh_gated_linear_scan: bad sizes");
     NVH_REQUIRE(dk <= 512, NVH_ENOSYS, "nvh_gated_linear_scan: key size %ld above 512", (long)dk);
     if (batch == 0) return NVH_OK;
     ScanArgs p{q, k, q_stride, k_stride, (int)qk_groups, w, w_stride, w_scalar, kscale, kscale_stride, v, v_stride, skip, state, slots,
-                     cu_seqlens_q, context_lens, out, (int)heads, (int)dk, (int)dv, 1, 1 << 30, ws_states, ws_decays};
+                     cu_seqlens_q, context_lens, out, (int)heads, (int)dk, (int)dv, 1, 1 << 30, ws_states, ws_decays, bonus};
+    NVH_REQUIRE(read_first || !bonus, NVH_EINVAL, "nvh_gated_linear_scan: a bonus needs read_first");
     if (segments > 1 && nvh_scan_segmentable(dk)) {
         NVH_REQUIRE(segments <= 64 && segment_min_tokens >= 2 * segments && ws_states && ws_decays && cu_seqlens_q, NVH_EINVAL, "nvh_gated_linear_scan: bad segments");
         p.nseg = (int)segments;
@@ -639,25 +779,25 @@ extern "C" int32_t nvh_gated_linear_scan(const float* q, int64_t q_stride, const
     // (the choice depends on dk alone, so a sequence sees one summation order whatever the batch or the cut)
     if (dk % 16 == 0) {
         switch (dk / 16) {
-            case 1: launch_scan_as<1, 16, true>(p, batch, st); break;
-            case 2: launch_scan_as<2, 16, true>(p, batch, st); break;
-            case 3: launch_scan_as<3, 16, true>(p, batch, st); break;
-            case 4: launch_scan_as<4, 16, true>(p, batch, st); break;
-            case 6: launch_scan_as<6, 16, true>(p, batch, st); break;
-            case 8: launch_scan_as<8, 16, true>(p, batch, st); break;
-            case 16: launch_scan_as<16, 16, true>(p, batch, st); break;
+            case 1: launch_scan_as<1, 16, true>(p, batch, read_first, st); break;
+            case 2: launch_scan_as<2, 16, true>(p, batch, read_first, st); break;
+            case 3: launch_scan_as<3, 16, true>(p, batch, read_first, st); break;
+            case 4: launch_scan_as<4, 16, true>(p, batch, read_first, st); break;
+            case 6: launch_scan_as<6, 16, true>(p, batch, read_first, st); break;
+            case 8: launch_scan_as<8, 16, true>(p, batch, read_first, st); break;
+            case 16: launch_scan_as<16, 16, true>(p, batch, read_first, st); break;
             default:
-                if (dk / 16 <= 8) launch_scan_as<8, 16, false>(p, batch, st);
-                else if (dk / 16 <= 16) launch_scan_as<16, 16, false>(p, batch, st);
-                else launch_scan_as<32, 16, false>(p, batch, st);
+                if (dk / 16 <= 8) launch_scan_as<8, 16, false>(p, batch, read_first, st);
+                else if (dk / 16 <= 16) launch_scan_as<16, 16, false>(p, batch, read_first, st);
+                else launch_scan_as<32, 16, false>(p, batch, read_first, st);
         }
     } else {
         const int dkq = (int)(dk + 3) / 4;
-        if (dkq <= 8) launch_scan_as<8, 4, false>(p, batch, st);
-        else if (dkq <= 16) launch_scan_as<16, 4, false>(p, batch, st);
-        else if (dkq <= 32) launch_scan_as<32, 4, false>(p, batch, st);
-        else if (dkq <= 64) launch_scan_as<64, 4, false>(p, batch, st);
-        else launch_scan_as<32, 16, false>(p, batch, st);
+        if (dkq <= 8) launch_scan_as<8, 4, false>(p, batch, read_first, st);
+        else if (dkq <= 16) launch_scan_as<16, 4, false>(p, batch, read_first, st);
+        else if (dkq <= 32) launch_scan_as<32, 4, false>(p, batch, read_first, st);
+        else if (dkq <= 64) launch_scan_as<64, 4, false>(p, batch, read_first, st);
+        else launch_scan_as<32, 16, false>(p, batch, read_first, st);
     }
     NVH_CHECK_LAUNCH("nvh_gated_linear_scan");
     return NVH_OK;
@@ -666,7 +806,7 @@ extern "C" int32_t nvh_gated_linear_scan(const float* q, int64_t q_stride, const
 extern "C" int32_t nvh_group_rmsnorm_gate(const float* o, const void* weight, int32_t weight_full, const void* gate, int64_t gate_stride,
                                           int32_t gate_act, int32_t gate_first, void* y, int64_t y_stride, int64_t rows, int64_t groups,
                                           int64_t group_size, float eps, int32_t act_f32, nvh_stream_t stream) {
-    NVH_REQUIRE(o && weight && y && rows >= 0 && groups > 0 && group_size > 0 && gate_act >= 0 && gate_act <= 2 && (!gate_act || gate), NVH_EINVAL,
+    NVH_REQUIRE(o && y && rows >= 0 && groups > 0 && group_size > 0 && gate_act >= 0 && gate_act <= 2 && (!gate_act || gate), NVH_EINVAL,
                 "nvh_group_rmsnorm_gate: bad argument");
     if (rows == 0) return NVH_OK;
     hipStream_t st = (hipStream_t)stream;

@@ -144,6 +144,169 @@ __global__ __launch_bounds__(256) void moe_route_linear_kernel(const A* __restri
         for (int r = 0; r < top; ++r) weights[t * top + r] = weights[t * top + r] / denom;
 }
 
+// Routing by scores: s = softmax(x W^T) over ALL experts; the choice goes by s + correction (a per-expert offset that
+// does not enter the weights), optionally restricted to groups of neighbouring experts - a group's score is its largest
+// choice score and only the `keep` best groups stay eligible (the others count as minus infinity); the `top` best eligible
+// experts are taken (ties: lower id) and weighted by their s times `scale`, not renormalised.  `aux` [n_aux, K]: further
+// rows that read the same input; their fp32 products go to aux_out [T, n_aux] (a gate of the layer, say).
+// One workgroup per token, products as in moe_route_linear_kernel; the first wave picks.
+template <typename A>
+__global__ __launch_bounds__(256) void moe_route_scored_kernel(const A* __restrict__ x, int64_t ldx, const A* __restrict__ w, const A* __restrict__ correction,
+                                                               const A* __restrict__ aux, float* __restrict__ aux_out, int n_aux, int32_t* __restrict__ ids,
+                                                               float* __restrict__ weights, float* __restrict__ scores_out, int experts, int K, int top,
+                                                               int groups, int keep, float scale, int vec) {
+    __shared__ float zs[64 * ROUTE_MAX_PER_LANE];            // logits, then scores
+    __shared__ float cs[64 * ROUTE_MAX_PER_LANE];            // choice scores
+    __shared__ float gsc[64 * ROUTE_MAX_PER_LANE];           // group scores
+    const int64_t t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const A* xr = x + t * ldx;
+    constexpr int EG = 4;
+    const int rows = experts + n_aux;
+    for (int e0 = wave * EG; e0 < rows; e0 += 4 * EG) {
+        float acc[EG];
+#pragma unroll
+        for (int g = 0; g < EG; ++g) acc[g] = 0.f;
+        for (int k0 = lane * 8; k0 < K; k0 += 512) {
+            float xv[8];
+            nvh_load8(xr, k0, K - k0, vec, xv);
+#pragma unroll
+            for (int g = 0; g < EG; ++g) {
+                const int e = min(e0 + g, rows - 1);
+                const A* wr = e < experts ? w + (int64_t)e * K : aux + (int64_t)(e - experts) * K;
+                float wv[8];
+                nvh_load8(wr, k0, K - k0, vec, wv);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc[g] = __builtin_fmaf(xv[i], wv[i], acc[g]);
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < EG; ++g) {
+            const int e = e0 + g;
+            const float sum = wave_sum(acc[g]);
+            if (lane == 0 && e < experts) zs[e] = sum;
+            else if (lane == 0 && e < rows) aux_out[t * n_aux + (e - experts)] = sum;
+        }
+    }
+    __syncthreads();
+    const bool picker = wave == 0;                           // the first wave picks; the others only keep the barriers company
+    // softmax over all experts
+    float z[ROUTE_MAX_PER_LANE];
+    if (picker) {
+        float mx = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j) {
+            z[j] = lane + 64 * j < experts ? zs[lane + 64 * j] : -INFINITY;
+            mx = fmaxf(mx, z[j]);
+        }
+        mx = wave_max(mx);
+        float den = 0.f;
+#pragma unroll
+        for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j) {
+            z[j] = lane + 64 * j < experts ? expf(z[j] - mx) : 0.f;
+            den += z[j];
+        }
+        den = wave_sum(den);
+#pragma unroll
+        for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j) {
+            const int e = lane + 64 * j;
+            if (e < experts) {
+                const float sc = z[j] / den;
+                zs[e] = sc;
+                if (scores_out) scores_out[t * experts + e] = sc;
+                z[j] = sc + (correction ? (float)correction[e] : 0.f);
+                cs[e] = z[j];
+            } else {
+                z[j] = -INFINITY;
+            }
+        }
+    }
+    __syncthreads();
+    if (groups > 1 && keep < groups) {                       // (uniform)
+        const int gsz = experts / groups;
+        float gv[ROUTE_MAX_PER_LANE];
+        bool gone[ROUTE_MAX_PER_LANE];
+        if (picker) {
+#pragma unroll
+            for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j) {
+                const int g = lane + 64 * j;
+                gone[j] = g >= groups;
+                gv[j] = -INFINITY;
+                if (g < groups) {
+                    for (int i = 0; i < gsz; ++i) gv[j] = fmaxf(gv[j], cs[g * gsz + i]);
+                    gsc[g] = 0.f;                            // becomes 1 for a kept group
+                }
+            }
+        }
+        __syncthreads();
+        if (picker) {
+            for (int r = 0; r < keep; ++r) {
+                float bv = -INFINITY;
+                int bg = 0x7fffffff;
+#pragma unroll
+                for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j)
+                    if (!gone[j] && (bg == 0x7fffffff || gv[j] > bv)) {
+                        bv = gv[j];
+                        bg = lane + 64 * j;
+                    }
+#pragma unroll
+                for (int off = 1; off < 64; off <<= 1) {
+                    const float ov = __shfl_xor(bv, off, 64);
+                    const int og = __shfl_xor(bg, off, 64);
+                    if (og != 0x7fffffff && (bg == 0x7fffffff || ov > bv || (ov == bv && og < bg))) {
+                        bv = ov;
+                        bg = og;
+                    }
+                }
+                if (lane == 0) gsc[bg] = 1.f;
+#pragma unroll
+                for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j)
+                    if (lane + 64 * j == bg) gone[j] = true;
+            }
+        }
+        __syncthreads();
+        if (picker) {
+#pragma unroll
+            for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j) {
+                const int e = lane + 64 * j;
+                if (e < experts && gsc[e / gsz] == 0.f) z[j] = -INFINITY;
+            }
+        }
+    }
+    if (!picker) return;
+    bool taken[ROUTE_MAX_PER_LANE];
+#pragma unroll
+    for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j) taken[j] = lane + 64 * j >= experts;
+    for (int r = 0; r < top; ++r) {
+        float bv = -INFINITY;
+        int be = 0x7fffffff;
+#pragma unroll
+        for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j) {
+            const int e = lane + 64 * j;
+            if (!taken[j] && (z[j] > bv || be == 0x7fffffff)) {
+                bv = z[j];
+                be = e;
+            }
+        }
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const float ov = __shfl_xor(bv, off, 64);
+            const int oe = __shfl_xor(be, off, 64);
+            if (oe != 0x7fffffff && (be == 0x7fffffff || ov > bv || (ov == bv && oe < be))) {
+                bv = ov;
+                be = oe;
+            }
+        }
+        if (lane == 0) {
+            ids[t * top + r] = be;
+            weights[t * top + r] = zs[be] * scale;
+        }
+#pragma unroll
+        for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j)
+            if (lane + 64 * j == be) taken[j] = true;
+    }
+}
+
 // One workgroup: counts per expert, block starts, then every pair takes the next free position of its expert's block.
 // (Which position a pair gets within its block depends on the order the lanes arrive in; nothing downstream depends on it.)
 __global__ __launch_bounds__(1024) void moe_align_kernel(const int32_t* __restrict__ ids, int64_t pairs, int experts, int top, int32_t* __restrict__ src_token,
@@ -224,15 +387,17 @@ __global__ __launch_bounds__(256) void gemm_grouped_f32_kernel(GroupedArgs a) {
 
 template <typename A>
 __global__ __launch_bounds__(256) void moe_combine_kernel(const A* __restrict__ y, int64_t ldy, const int32_t* __restrict__ pos_of_pair, const float* __restrict__ weights,
-                                                          const A* __restrict__ shared, int64_t shared_stride, float* __restrict__ out, int dim, int top) {
+                                                          const A* __restrict__ shared, int64_t shared_stride, const float* __restrict__ shared_gate,
+                                                          int64_t gate_stride, float* __restrict__ out, int dim, int top) {
     const int64_t t = blockIdx.x;
+    const float sg = shared_gate ? 1.0f / (1.0f + expf(-shared_gate[t * gate_stride])) : 1.0f;
     for (int c = threadIdx.x; c < dim; c += 256) {
         float s = 0.f;
         for (int r = 0; r < top; ++r) {
             const int pos = pos_of_pair[t * top + r];
             if (pos >= 0) s = __builtin_fmaf(weights[t * top + r], (float)y[(int64_t)pos * ldy + c], s);
         }
-        if (shared) s += (float)shared[t * shared_stride + c];
+        if (shared) s += sg * (float)shared[t * shared_stride + c];
         out[t * dim + c] = s;
     }
 }
@@ -263,6 +428,25 @@ extern "C" int32_t nvh_moe_route_linear(const void* x, int64_t x_row_stride, con
     if (act_f32) moe_route_linear_kernel<float><<<grid, 256, 0, st>>>((const float*)x, x_row_stride, (const float*)w, (const float*)bias, ids, weights, logits_out, (int)experts, (int)K, (int)top, vec);
     else moe_route_linear_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)x, x_row_stride, (const bf16*)w, (const bf16*)bias, ids, weights, logits_out, (int)experts, (int)K, (int)top, vec);
     NVH_CHECK_LAUNCH("nvh_moe_route_linear");
+    return NVH_OK;
+}
+
+extern "C" int32_t nvh_moe_route_scored(const void* x, int64_t x_row_stride, const void* w, const void* correction, const void* aux, float* aux_out,
+                                        int64_t num_aux, int32_t* ids, float* weights, float* scores_out, int64_t num_tokens, int64_t experts, int64_t K,
+                                        int64_t top, int64_t groups, int64_t keep, float scale, int32_t act_f32, nvh_stream_t stream) {
+    NVH_REQUIRE(x && w && ids && weights && (num_aux == 0 || (aux && aux_out)), NVH_EINVAL, "nvh_moe_route_scored: null pointer");
+    NVH_REQUIRE(num_tokens >= 0 && experts > 0 && top > 0 && top <= experts && K > 0 && K < (1 << 30) && x_row_stride >= K && num_aux >= 0 && num_aux <= 64, NVH_EINVAL,
+                "nvh_moe_route_scored: bad sizes");
+    NVH_REQUIRE(groups >= 1 && experts % groups == 0 && keep >= 1 && keep <= groups && top <= keep * (experts / groups), NVH_EINVAL,
+                "nvh_moe_route_scored: %ld groups (keep %ld) do not fit %ld experts, top %ld", (long)groups, (long)keep, (long)experts, (long)top);
+    NVH_REQUIRE(experts <= 64 * ROUTE_MAX_PER_LANE, NVH_ENOSYS, "nvh_moe_route_scored: %ld experts above %d", (long)experts, 64 * ROUTE_MAX_PER_LANE);
+    if (num_tokens == 0) return NVH_OK;
+    const dim3 grid((unsigned)num_tokens);
+    hipStream_t st = (hipStream_t)stream;
+    const int vec = K % 8 == 0 && x_row_stride % 8 == 0 && nvh_aligned16(x) && nvh_aligned16(w) && (!aux || nvh_aligned16(aux));
+    if (act_f32) moe_route_scored_kernel<float><<<grid, 256, 0, st>>>((const float*)x, x_row_stride, (const float*)w, (const float*)correction, (const float*)aux, aux_out, (int)num_aux, ids, weights, scores_out, (int)experts, (int)K, (int)top, (int)groups, (int)keep, scale, vec);
+    else moe_route_scored_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)x, x_row_stride, (const bf16*)w, (const bf16*)correction, (const bf16*)aux, aux_out, (int)num_aux, ids, weights, scores_out, (int)experts, (int)K, (int)top, (int)groups, (int)keep, scale, vec);
+    NVH_CHECK_LAUNCH("nvh_moe_route_scored");
     return NVH_OK;
 }
 
@@ -301,12 +485,13 @@ extern "C" int32_t nvh_gemm_grouped_any_nt(const void* x, int64_t x_row_stride, 
 }
 
 extern "C" int32_t nvh_moe_combine(const void* y, int64_t y_row_stride, const int32_t* pos_of_pair, const float* weights, const void* shared,
-                                   int64_t shared_stride, float* out, int64_t num_tokens, int64_t dim, int64_t top, int32_t act_f32, nvh_stream_t stream) {
+                                   int64_t shared_stride, const float* shared_gate, int64_t shared_gate_stride, float* out, int64_t num_tokens, int64_t dim,
+                                   int64_t top, int32_t act_f32, nvh_stream_t stream) {
     NVH_REQUIRE(y && pos_of_pair && weights && out && num_tokens >= 0 && dim > 0 && top > 0 && y_row_stride >= dim, NVH_EINVAL, "nvh_moe_combine: bad argument");
     if (num_tokens == 0) return NVH_OK;
     hipStream_t st = (hipStream_t)stream;
-    if (act_f32) moe_combine_kernel<float><<<dim3((unsigned)num_tokens), 256, 0, st>>>((const float*)y, y_row_stride, pos_of_pair, weights, (const float*)shared, shared_stride, out, (int)dim, (int)top);
-    else moe_combine_kernel<bf16><<<dim3((unsigned)num_tokens), 256, 0, st>>>((const bf16*)y, y_row_stride, pos_of_pair, weights, (const bf16*)shared, shared_stride, out, (int)dim, (int)top);
+    if (act_f32) moe_combine_kernel<float><<<dim3((unsigned)num_tokens), 256, 0, st>>>((const float*)y, y_row_stride, pos_of_pair, weights, (const float*)shared, shared_stride, shared_gate, shared_gate_stride, out, (int)dim, (int)top);
+    else moe_combine_kernel<bf16><<<dim3((unsigned)num_tokens), 256, 0, st>>>((const bf16*)y, y_row_stride, pos_of_pair, weights, (const bf16*)shared, shared_stride, shared_gate, shared_gate_stride, out, (int)dim, (int)top);
     NVH_CHECK_LAUNCH("nvh_moe_combine");
     return NVH_OK;
 }

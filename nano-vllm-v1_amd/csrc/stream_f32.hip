@@ -234,8 +234,60 @@ __global__ __launch_bounds__(256) void residual_norm_kernel(CloseArgs p) {
     }
 }
 
+// The close of a sublayer in a stack that norms AFTER the sum, per row:
+//   v = alpha x + ls (y + y32);   x <- v rsqrt(mean(v^2) + eps) (offset + w);   h <- x in the activation type
+// alpha: the weight of the old stream in the sum; ls: a per-column scale of the sublayer's result (null: 1); y (type A) and
+// y32 (fp32) are the sublayer's result, either or both may be absent (none: the norm alone, with alpha; write_x 0 then leaves
+// the stream as it is and gives h only).  offset 1 serves
+// a weight that is stored around zero.  The stream stays fp32; the sum, the statistics and the product are fp32.
+struct PostNormArgs {
+    const void* y;
+    int64_t y_stride;
+    const float* y32;
+    int64_t y32_stride;
+    const void* ls;
+    float alpha;
+    float* x;
+    const void* nw;
+    float offset, eps;
+    void* h;
+    int64_t h_stride;
+    int dim, write_x;
+};
+
+template <typename A>
+__global__ __launch_bounds__(256) void residual_postnorm_kernel(PostNormArgs p) {
+    extern __shared__ float rowbuf[];
+    __shared__ float red[4];
+    const int64_t row = blockIdx.x;
+    const int dim = p.dim;
+    const A* y = p.y ? (const A*)p.y + row * p.y_stride : nullptr;
+    const float* y32 = p.y32 ? p.y32 + row * p.y32_stride : nullptr;
+    const A* ls = (const A*)p.ls;
+    float* xr = p.x + row * dim;
+    float sq = 0.f;
+    for (int i = threadIdx.x; i < dim; i += 256) {
+        float v = p.alpha * xr[i];
+        if (y || y32) {
+            float s = y ? (float)y[i] : 0.f;
+            if (y32) s += y32[i];
+            if (ls) s *= (float)ls[i];
+            v += s;
+        }
+        rowbuf[i] = v;
+        sq += v * v;
+    }
+    const float inv = 1.0f / sqrtf(block_sum4(sq, red) / (float)dim + p.eps);
+    A* h = p.h ? (A*)p.h + row * p.h_stride : nullptr;
+    for (int i = threadIdx.x; i < dim; i += 256) {
+        const float v = rowbuf[i] * inv * (p.offset + (float)((const A*)p.nw)[i]);
+        if (p.write_x) xr[i] = v;
+        if (h) h[i] = (A)v;
+    }
+}
+
 // y = act(g) (* u when gated): g = columns [0, inter) and u = columns [inter, 2 inter) of the row.
-// act: 0 silu, 1 gelu (tanh form), 2 squared relu.
+// act: 0 silu, 1 gelu (tanh form), 2 squared relu, 3 tanh.
 template <typename A>
 __global__ __launch_bounds__(256) void act_mul_kernel(const A* __restrict__ gu, int64_t gu_stride, A* __restrict__ y, int64_t y_stride, int64_t rows, int inter,
                                                       int act, int gated) {
@@ -247,7 +299,8 @@ __global__ __launch_bounds__(256) void act_mul_kernel(const A* __restrict__ gu, 
     float v;
     if (act == 0) v = g / (1.0f + expf(-g));
     else if (act == 1) v = 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
-    else v = g > 0.f ? g * g : 0.f;
+    else if (act == 2) v = g > 0.f ? g * g : 0.f;
+    else v = tanhf(g);
     if (gated) v *= ldf(gu, row * gu_stride + inter + c);
     y[row * y_stride + c] = (A)v;
 }
@@ -414,9 +467,29 @@ extern "C" int32_t nvh_residual_norm(const void* a, int64_t a_stride, const void
     return NVH_OK;
 }
 
+extern "C" int32_t nvh_residual_postnorm(const void* y, int64_t y_stride, const float* y32, int64_t y32_stride, const void* layer_scale, float alpha,
+                                         float* x, int32_t write_x, const void* norm_weight, float weight_offset, float eps, void* h, int64_t h_stride,
+                                         int64_t rows, int64_t dim, int32_t act_f32, nvh_stream_t stream) {
+    NVH_STREAM_ARGS_OK("nvh_residual_postnorm", x && norm_weight && rows >= 0 && dim > 0 && dim <= 32768 && (!y || y_stride >= dim) && (!y32 || y32_stride >= dim) &&
+                                                    (!h || h_stride >= dim));
+    if (rows == 0) return NVH_OK;
+    const PostNormArgs p{y, y_stride, y32, y32_stride, layer_scale, alpha, x, norm_weight, weight_offset, eps, h, h_stride, (int)dim, write_x};
+    hipStream_t st = (hipStream_t)stream;
+    const size_t lds = sizeof(float) * (size_t)dim;
+    if (lds > 48 * 1024) {
+        const hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(&residual_postnorm_kernel<float>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        const hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(&residual_postnorm_kernel<bf16>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        NVH_REQUIRE(e1 == hipSuccess && e2 == hipSuccess, NVH_ENOSYS, "nvh_residual_postnorm: %zu bytes of LDS refused", lds);
+    }
+    if (act_f32) residual_postnorm_kernel<float><<<dim3((unsigned)rows), 256, lds, st>>>(p);
+    else residual_postnorm_kernel<bf16><<<dim3((unsigned)rows), 256, lds, st>>>(p);
+    NVH_CHECK_LAUNCH("nvh_residual_postnorm");
+    return NVH_OK;
+}
+
 extern "C" int32_t nvh_act_mul(const void* x, int64_t row_stride, void* y, int64_t y_stride, int64_t rows, int64_t inter, int32_t act, int32_t gated,
                                int32_t act_f32, nvh_stream_t stream) {
-    NVH_STREAM_ARGS_OK("nvh_act_mul", x && y && rows >= 0 && inter > 0 && act >= 0 && act <= 2 && row_stride >= (gated ? 2 : 1) * inter && y_stride >= inter);
+    NVH_STREAM_ARGS_OK("nvh_act_mul", x && y && rows >= 0 && inter > 0 && act >= 0 && act <= 3 && row_stride >= (gated ? 2 : 1) * inter && y_stride >= inter);
     if (rows == 0) return NVH_OK;
     hipStream_t st = (hipStream_t)stream;
     const unsigned blocks = (unsigned)nvh_cdiv(rows * inter, 256);

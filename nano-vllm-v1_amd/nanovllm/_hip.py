@@ -105,13 +105,16 @@ SIGNATURES = {
     # layer norm / RMS norm around the fp32 stream, plain activations (csrc/stream_f32.hip)
     "nvh_embedding_pos_stream": (i32, [vp, vp, vp, vp, f32, vp, i64, i64, i64, i64, i32, vp]),
     "nvh_residual_norm": (i32, [vp, i64, vp, vp, i64, vp, f32, f32, vp, i64, vp, i64, vp, i32, vp, vp, f32, vp, i64, i64, i64, i32, vp]),
+    "nvh_residual_postnorm": (i32, [vp, i64, vp, i64, vp, f32, vp, i32, vp, f32, f32, vp, i64, i64, i64, i32, vp]),
     "nvh_act_mul": (i32, [vp, i64, vp, i64, i64, i64, i32, i32, i32, vp]),
     "nvh_logits_scale": (i32, [vp, i64, vp, i64, i64, f32, f32, i32, vp]),
     # linear recurrences with a diagonal decay (csrc/linear_recurrence.hip)
-    "nvh_gated_linear_scan": (i32, [vp, i64, vp, i64, i64, vp, i64, i32, vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, vp, vp]),
+    "nvh_gated_linear_scan": (i32, [vp, i64, vp, i64, i64, vp, i64, i32, vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, vp, i32, vp, vp]),
     "nvh_scan_segmentable": (i32, [i64]),
     "nvh_hgrn2_prep": (i32, [vp, i64, vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, i64, i64, i64, i32, vp]),
-    "nvh_gla_prep": (i32, [vp, i64, vp, i64, vp, i64, vp, i64, f32, f32, vp, vp, vp, vp, i64, i64, i64, i32, vp]),
+    "nvh_gla_prep": (i32, [vp, i64, vp, i64, vp, i64, vp, i64, f32, f32, vp, vp, vp, vp, i64, i64, i64, i32, i32, vp]),
+    "nvh_token_shift_mix": (i32, [vp, i64, vp, vp, vp, vp, i64, vp, vp, i64, i64, i64, i32, vp]),
+    "nvh_rotary_qkv_prep": (i32, [vp, i64, vp, i64, vp, i64, vp, vp, f32, i64, i32, f32, f32, vp, vp, vp, i64, i64, i64, i64, i32, vp]),
     "nvh_ssd_conv_prep": (i32, [vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, vp, vp, vp, vp, i32, vp]),
     "nvh_conv_state_update": (i32, [vp, i64, vp, vp, vp, vp, i64, i64, i64, i32, vp]),
     "nvh_group_rmsnorm_gate": (i32, [vp, vp, i32, vp, i64, i32, i32, vp, i64, i64, i64, i64, f32, i32, vp]),
@@ -121,7 +124,12 @@ SIGNATURES = {
     "nvh_moe_max_tiles": (i64, [i64, i64]),
     "nvh_moe_align": (i32, [vp, i64, i64, i64, vp, vp, vp, vp, vp, i64, vp]),
     "nvh_gemm_grouped_any_nt": (i32, [vp, i64, vp, vp, vp, i64, vp, vp, vp, i64, i64, i64, i32, i32, vp]),
-    "nvh_moe_combine": (i32, [vp, i64, vp, vp, vp, i64, vp, i64, i64, i64, i32, vp]),
+    "nvh_moe_combine": (i32, [vp, i64, vp, vp, vp, i64, vp, i64, vp, i64, i64, i64, i32, vp]),
+    "nvh_moe_route_scored": (i32, [vp, i64, vp, vp, vp, vp, i64, vp, vp, vp, i64, i64, i64, i64, i64, i64, f32, i32, vp]),
+    # attention through a low-rank latent (csrc/latent_attention.hip)
+    "nvh_latent_prep": (i32, [vp, i64, i64, i64, i64, i64, i32, vp, vp, f32, vp, vp, f32, i32, vp, vp, vp, vp, vp, i64, i64, i32, vp]),
+    "nvh_latent_q_rotary": (i32, [vp, i64, vp, vp, f32, i32, vp, i64, i64, i64, i64, i64, i64, i64, i32, vp]),
+    "nvh_gemm_heads_nt": (i32, [vp, i64, i64, vp, vp, i64, i64, i64, i64, i64, i64, i32, vp]),
 }
 
 _lib = None

@@ -405,10 +405,12 @@ class ModelRunner:
         read, and a sequence's state is taken as zero in the step that brings its first tokens."""
         paged, recurrent = self._cache_modules()
         for m in paged:
+            # (key/value heads, key size, value size) of a cached token: named by the module, or its plain head sizes
+            g, dk, dv = m.cache_geometry() if hasattr(m, "cache_geometry") else (m.num_kv_heads, m.head_dim, m.value_dim)
             for run in range(m.cache_runs):
                 if num_blocks:
-                    m.k_caches[run] = torch.zeros(num_blocks, self.block_size, m.num_kv_heads, m.head_dim, dtype=self.dtype, device=self.device)
-                    m.v_caches[run] = torch.zeros(num_blocks, m.num_kv_heads, m.value_dim, self.block_size, dtype=self.dtype, device=self.device)
+                    m.k_caches[run] = torch.zeros(num_blocks, self.block_size, g, dk, dtype=self.dtype, device=self.device)
+                    m.v_caches[run] = torch.zeros(num_blocks, g, dv, self.block_size, dtype=self.dtype, device=self.device)
                 else:
                     m.k_caches[run] = m.v_caches[run] = None
         for m in recurrent:

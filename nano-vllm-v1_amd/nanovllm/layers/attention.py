@@ -149,3 +149,84 @@ class WindowedBiasAttention(nn.Module):
         return ops.attn_paged_any(q, kc, vc, ctx.cu_seqlens_q, ctx.context_lens, ctx.block_tables, self.scale, self.num_heads,
                                   self.num_kv_heads, self.head_dim, self.value_dim, slopes=self.slopes, window=self.window,
                                   keep_first=self.keep_first)
+
+
+class LatentAttention(nn.Module):
+    """Causal softmax attention whose keys and values are read from a low-rank latent ("DeepSeek-V2: A Strong, Economical, and Efficient
+    Mixture-of-Experts Language Model", DeepSeek-AI): a token leaves in the cache only its RMS-normed latent c (`kv_rank` wide) and
+    one rotated key part k_r (`rot_dim` wide) that all heads share; head h's unrotated key is W_uk,h c and its value W_uv,h c.  Both are
+    linear in c, so they are never formed: the query side takes W_uk in,
+
+        score = scale ((W_uk,h^T q_n) . c + q_r . k_r),      out_h = W_uv,h (sum_j p_j c_j),
+
+    which is paged attention of H query heads over ONE shared key/value head of key size kv_rank + rot_dim whose value is c
+    (nvh_attn_paged_any), between two per-head products (nvh_gemm_heads_nt).  The query itself comes through a latent too
+    (RMS-normed, `q_rank` wide) and is laid out per head as [dim unrotated | rot_dim rotated]; an optional sigmoid gate per head
+    scales the head's output.
+
+    Input of forward: the fused projection row [dq | dkv | gate] of the layer's input.  A module built with `kv_source` owns no
+    cache and has no dkv part: it reads the latent and rotated key part that the source module cached for the same tokens (the
+    source runs earlier in the step), with its own W_uk, W_uv and queries.  `uq` maps the normed query latent to the heads."""
+
+    def __init__(self, num_heads: int, head_dim: int, rot_dim: int, value_dim: int, q_rank: int, kv_rank: int, scale: float, eps: float,
+                 freq: torch.Tensor | None, mag: float = 1.0, interleaved: bool = True, gated: bool = True, cache_runs: int = 1,
+                 kv_source: "LatentAttention | None" = None):
+        super().__init__()
+        from .linear import MergedLinear
+        self.num_heads, self.qk_dim, self.rot_dim, self.v_dim, self.q_rank, self.kv_rank = num_heads, head_dim, rot_dim, value_dim, q_rank, kv_rank
+        self.scale, self.eps, self.mag, self.interleaved, self.gated = scale, eps, mag, interleaved, gated
+        self.q_norm = nn.Parameter(torch.ones(q_rank), requires_grad=False)
+        self.uq = MergedLinear(q_rank, [num_heads * (head_dim + rot_dim)])
+        # W_uk is stored transposed per head ([H, kv_rank, dim]): it multiplies the query, not the latent
+        self.uk_t = nn.Parameter(torch.empty(num_heads, kv_rank, head_dim), requires_grad=False)
+        self.uk_t.weight_loader = self._load_uk
+        self.uv = nn.Parameter(torch.empty(num_heads, value_dim, kv_rank), requires_grad=False)
+        self.uv.weight_loader = self._load_uv
+        self.register_buffer("freq", None if freq is None else freq.to(dtype=torch.float32, device=self.q_norm.device), persistent=False)
+        self._source = [kv_source] if kv_source is not None else None       # (a list: the source is not a submodule of this one)
+        if kv_source is None:
+            self.kv_norm = nn.Parameter(torch.ones(kv_rank), requires_grad=False)
+            self.cache_runs = cache_runs
+            self.k_caches: list = [None] * cache_runs
+            self.v_caches: list = [None] * cache_runs
+        else:
+            assert (kv_source.kv_rank, kv_source.rot_dim) == (kv_rank, rot_dim) and kv_source._source is None, "the source of a shared latent must own one of the same sizes"
+            self.register_parameter("kv_norm", None)
+
+    def _load_uk(self, param: nn.Parameter, loaded_weight: torch.Tensor):
+        assert tuple(loaded_weight.shape) == (self.num_heads * self.qk_dim, self.kv_rank), tuple(loaded_weight.shape)
+        param.data.copy_(loaded_weight.view(self.num_heads, self.qk_dim, self.kv_rank).transpose(1, 2))
+
+    def _load_uv(self, param: nn.Parameter, loaded_weight: torch.Tensor):
+        assert tuple(loaded_weight.shape) == (self.num_heads * self.v_dim, self.kv_rank), tuple(loaded_weight.shape)
+        param.data.copy_(loaded_weight.view(self.num_heads, self.v_dim, self.kv_rank))
+
+    # what the runner sizes and shapes the page pool with (modules without caches of their own are not asked)
+    def cache_geometry(self) -> tuple[int, int, int]:
+        """(key/value heads, key size, value size) of a cached token."""
+        return 1, self.kv_rank + self.rot_dim, self.kv_rank
+
+    def cache_row_elems(self) -> tuple[int, int]:
+        return self.kv_rank + self.rot_dim, self.kv_rank
+
+    def projection_sizes(self) -> list[int]:
+        own = [] if self._source is not None else [self.kv_rank + self.rot_dim]
+        return [self.q_rank] + own + ([self.num_heads] if self.gated else [])
+
+    def forward(self, proj: torch.Tensor, positions: torch.Tensor, run: int = 0) -> torch.Tensor:
+        ctx = get_context()
+        owner = self if self._source is None else self._source[0]
+        kc, vc = owner.k_caches[run], owner.v_caches[run]
+        if kc is None or ctx.block_tables is None:
+            raise RuntimeError("this attention reads its keys from the paged cache: bind caches and give every sequence a block table")
+        own = self._source is None
+        cq, gate = ops.latent_prep(proj, self.q_rank, self.kv_rank, self.rot_dim, self.num_heads, self.q_norm.data, self.kv_norm.data if own else None,
+                                   self.eps, positions, self.freq, self.mag, self.interleaved, kc if own else None, vc if own else None,
+                                   ctx.slot_mapping if own else None, self.gated)
+        q = self.uq(cq)                                                     # [T, H * (dim + rot)]
+        t, full = q.shape[0], self.kv_rank + self.rot_dim
+        qa = torch.empty(t, self.num_heads * full, dtype=q.dtype, device=q.device)
+        ops.linear_heads(q, self.uk_t.data, self.qk_dim + self.rot_dim, out=qa, out_head_stride=full)
+        ops.latent_q_rotary(q, positions, self.freq, self.mag, self.interleaved, qa, self.num_heads, self.qk_dim, self.rot_dim, full, self.kv_rank)
+        o = ops.attn_paged_any(qa, kc, vc, ctx.cu_seqlens_q, ctx.context_lens, ctx.block_tables, self.scale, self.num_heads, 1, full, self.kv_rank, gate)
+        return ops.linear_heads(o, self.uv.data, self.kv_rank)

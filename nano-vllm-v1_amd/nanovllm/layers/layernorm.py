@@ -3,6 +3,8 @@ StreamNorm: a layer norm or RMS norm of the fp32 residual stream, applied togeth
 nvh_residual_norm (csrc/stream_f32.hip).
 DynamicTanh: a norm without statistics, tanh(alpha x) * weight + bias, applied together with the residual add around
 it by nvh_residual_dyt (csrc/stream_f32.hip) over an fp32 residual stream.
+PostSumRMSNorm: an RMS norm taken AFTER the residual sum (the stream itself is the normed value), with the old stream's
+weight in the sum, a per-column scale of the sublayer's result and a weight stored around zero (nvh_residual_postnorm).
 
 Interface of the reference's nanovllm/layers/layernorm.py:48-165: ``RMSNorm(hidden_size,
 eps)``, ``.weight``, ``forward(x)`` -> y, ``forward(x, residual)`` -> (y, new_residual).
@@ -74,3 +76,31 @@ class StreamNorm(nn.Module):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         """x fp32 [rows, dim] -> normalised rows in the parameters' type (x is left as it is)."""
         return ops.residual_norm(x, **self.spec())
+
+
+class PostSumRMSNorm(nn.Module):
+    """The close of a sublayer in a stack that norms after the sum:
+
+        x <- rms_norm(alpha x + scale * sublayer(x)) * (offset + weight)
+
+    alpha weighs the old stream in the sum, `scale` (one factor per column, optional) the sublayer's result, and `offset` = 1
+    serves a weight that is stored around zero.  The stream x is fp32 and is replaced in place; `close` returns it once
+    more in the activation type, the input of the next sublayer."""
+
+    def __init__(self, hidden_size: int, eps: float, alpha: float = 1.0, weight_offset: float = 0.0, layer_scale: bool = False) -> None:
+        super().__init__()
+        self.eps, self.alpha, self.weight_offset = eps, float(alpha), float(weight_offset)
+        self.weight = nn.Parameter(torch.zeros(hidden_size) if weight_offset else torch.ones(hidden_size), requires_grad=False)
+        if layer_scale:
+            self.scale = nn.Parameter(torch.ones(hidden_size), requires_grad=False)
+        else:
+            self.register_parameter("scale", None)
+
+    def close(self, x: torch.Tensor, y: torch.Tensor | None = None, y32: torch.Tensor | None = None, want_h: bool = True):
+        """y: the sublayer's result in the activation type, y32: in fp32 (either, both or none)."""
+        return ops.residual_postnorm(x, self.weight.data, self.eps, y, y32, None if self.scale is None else self.scale.data, self.alpha,
+                                     self.weight_offset, want_h)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """The norm alone (no sum, the stream taken once): x fp32 [rows, dim] -> normed rows in the activation type (x is left as it is)."""
+        return ops.residual_postnorm(x, self.weight.data, self.eps, None, None, None, 1.0, self.weight_offset, True, in_place=False)

@@ -4,6 +4,13 @@
     picked = the `top` largest z; weights = softmax taken over those `top` values only
     y = sum_picked weight_e * down_e(act(gate_e h) * up_e h)  (+ shared(h), a gated feed-forward every token passes)
 
+or, with score="softmax_all" (the routing of "DeepSeek-V3 Technical Report", DeepSeek-AI, with softmax scores):
+
+    s = softmax(W_router h) over all experts;  the choice goes by s + correction (a per-expert offset that never enters the weights),
+    restricted to the `keep` best of `groups` equal groups of neighbouring experts (a group's score: its largest corrected score);
+    picked = the `top` best eligible;  weights = route_scale * s[picked], not renormalised;
+    the shared expert's result is multiplied by sigmoid(W_sg h), one number per token (shared_gate=True).
+
 The experts' matrices lie stacked, gate and up merged ([E, 2 ff, D] and [E, D, ff]), and run as two grouped products over
 the (token, choice) pairs ordered by expert (ops.moe_align / ops.linear_grouped); routing, ordering and the tile list stay on
 the device, so a step with experts needs no answer from the host and can be captured in a graph.  The result is the fp32
@@ -33,11 +40,23 @@ class GatedMLP(nn.Module):
 
 
 class SparseMoE(nn.Module):
-    def __init__(self, width: int, ff: int, experts: int, top: int, shared_ff: int | None = None, act: str = "silu", router_bias: bool = True):
+    def __init__(self, width: int, ff: int, experts: int, top: int, shared_ff: int | None = None, act: str = "silu", router_bias: bool = True,
+                 score: str = "softmax_top", correction: bool = False, groups: int = 1, keep_groups: int = 1, route_scale: float = 1.0,
+                 shared_gate: bool = False):
         super().__init__()
-        assert 1 <= top <= experts
-        self.width, self.ff, self.experts, self.top, self.act = width, ff, experts, top, act
+        assert 1 <= top <= experts and score in ("softmax_top", "softmax_all")
+        self.width, self.ff, self.experts, self.top, self.act, self.score = width, ff, experts, top, act, score
+        self.groups, self.keep_groups, self.route_scale = int(groups), int(keep_groups), float(route_scale)
+        if score == "softmax_all":
+            assert not router_bias and experts % self.groups == 0 and 1 <= self.keep_groups <= self.groups
+            assert top <= self.keep_groups * (experts // self.groups), "fewer eligible experts than choices"
+        else:
+            assert not correction and self.groups == 1 and route_scale == 1.0, "these options belong to score='softmax_all'"
         self.router = MergedLinear(width, [experts], bias=router_bias)
+        if correction:
+            self.correction = nn.Parameter(torch.zeros(experts), requires_grad=False)
+        else:
+            self.register_parameter("correction", None)
         self.gate_up = nn.Parameter(torch.empty(experts, 2 * ff, width), requires_grad=False)
         self.down = nn.Parameter(torch.empty(experts, width, ff), requires_grad=False)
         self.gate_up.weight_loader = self._load_gate_up
@@ -45,6 +64,7 @@ class SparseMoE(nn.Module):
         self.gate_up.shard_ids = [(e, part) for e in range(experts) for part in ("gate", "up")]
         self.down.shard_ids = list(range(experts))
         self.shared = GatedMLP(width, shared_ff, act) if shared_ff else None
+        self.shared_gate = MergedLinear(width, [1]) if (shared_gate and shared_ff) else None      # one logit per token
 
     def _load_gate_up(self, param: nn.Parameter, loaded_weight: torch.Tensor, shard_id):
         e, part = shard_id
@@ -58,8 +78,16 @@ class SparseMoE(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         """x [T, width] in the activation type -> fp32 [T, width]."""
-        ids, weights = ops.moe_route_linear(x, self.router.weight.data, None if self.router.bias is None else self.router.bias.data, self.top)
+        gate = None
+        if self.score == "softmax_all":
+            ids, weights, gate = ops.moe_route_scored(x, self.router.weight.data, self.top, None if self.correction is None else self.correction.data,
+                                                      self.groups, self.keep_groups, self.route_scale,
+                                                      aux=None if self.shared_gate is None else self.shared_gate.weight.data)
+        else:
+            ids, weights = ops.moe_route_linear(x, self.router.weight.data, None if self.router.bias is None else self.router.bias.data, self.top)
+            if self.shared_gate is not None:
+                gate = self.shared_gate(x, out_f32=True)
         plan = ops.moe_align(ids, self.experts)
         hidden = ops.act_mul(ops.linear_grouped(x, self.gate_up.data, plan, gather=True), self.act, True)
         y = ops.linear_grouped(hidden, self.down.data, plan, gather=False)
-        return ops.moe_combine(y, plan, weights, self.shared(x) if self.shared is not None else None)
+        return ops.moe_combine(y, plan, weights, self.shared(x) if self.shared is not None else None, gate)

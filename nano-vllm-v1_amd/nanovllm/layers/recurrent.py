@@ -78,7 +78,9 @@ class DiagonalDecayRecurrence(_StatePool):
         S <- diag(w) S + (c k) v^T,      o = S^T q + d v
 
     w: one decay for each key channel, or a single one per head, c: a write strength per head (None: 1), d: a skip weight per head (None: 0),
-    q and k possibly shared by groups of heads.  The operands are fp32 (the mixers below make them from their projections);
+    q and k possibly shared by groups of heads.  `read_first`: the token is read out before it is written and the state
+    decayed, with a bonus u per head and key channel for the token itself, o = (S + diag(u) (c k) v^T)^T q + d v (the RWKV
+    time mix).  The operands are fp32 (the mixers below make them from their projections);
     the scan walks this step's tokens of every sequence from the state its slot holds, or from zero when the sequence
     starts in this step (kernel: nvh_gated_linear_scan, csrc/linear_recurrence.hip)."""
 
@@ -86,11 +88,12 @@ class DiagonalDecayRecurrence(_StatePool):
         super().__init__((num_heads, value_dim, key_dim), state_runs)      # stored transposed: a column's key rows lie together
         self.num_heads, self.key_dim, self.value_dim, self.qk_groups = num_heads, key_dim, value_dim, qk_groups or num_heads
 
-    def forward(self, q, k, w, v, run: int = 0, kscale=None, skip=None) -> torch.Tensor:
+    def forward(self, q, k, w, v, run: int = 0, kscale=None, skip=None, read_first: bool = False, bonus=None) -> torch.Tensor:
         state = self.pool(run)
         ctx = get_context()
         return ops.gated_linear_scan(q, k, w, v, state, ctx.state_slots, ctx.cu_seqlens_q, ctx.context_lens, self.num_heads, self.key_dim,
-                                     self.value_dim, self.qk_groups, kscale, skip, max_seqlen_q=ctx.max_seqlen_q or 0)
+                                     self.value_dim, self.qk_groups, kscale, skip, max_seqlen_q=ctx.max_seqlen_q or 0, read_first=read_first,
+                                     bonus=bonus)
 
 
 class HGRN2(nn.Module):
@@ -168,3 +171,76 @@ class Mamba2(nn.Module):
                                                  self.num_heads, self.inner, self.gn)
         y = self.memory(c, b, decay, x, run, kscale=step, skip=self.D.data)
         return ops.group_rmsnorm_gate(y, self.norm.data, self.inner // self.norm_groups, self.eps, z, "silu", gate_first=True)
+
+
+class Retention(nn.Module):
+    """Retention: linear attention with one fixed decay per head and neither softmax nor denominator.  Per head, with rotary
+    positions on the first `rot_dims` dimensions of q and k (frequencies given by the caller; pairs in halves unless
+    `interleaved`) and k scaled by key_dim^(-1/2) after the rotation:
+
+        S <- decay_h S + k v^T,      o = S^T q
+
+    The read-out of a head is divided by its root mean square (no weight) and multiplied by silu(gate).
+
+    forward takes the column views q, k, v, gate of the fused projection and returns [T, H * value_dim] in the activation type."""
+
+    def __init__(self, num_heads: int, key_dim: int, value_dim: int, decays, eps: float, rot_dims: int = 0, freq: torch.Tensor | None = None,
+                 mag: float = 1.0, interleaved: bool = False, state_runs: int = 1):
+        super().__init__()
+        decays = torch.as_tensor(decays, dtype=torch.float64).to(torch.float32)
+        assert decays.numel() == num_heads and 0 <= rot_dims <= key_dim and rot_dims % 2 == 0
+        self.num_heads, self.key_dim, self.value_dim, self.eps = num_heads, key_dim, value_dim, eps
+        self.rot_dims, self.mag, self.interleaved = rot_dims, mag, interleaved
+        dev = torch.empty(0).device
+        self.register_buffer("decays", decays.to(dev), persistent=False)
+        self.register_buffer("freq", None if freq is None else freq.to(dtype=torch.float32, device=dev), persistent=False)
+        self.memory = DiagonalDecayRecurrence(num_heads, key_dim, value_dim, state_runs=state_runs)
+
+    def forward(self, q, k, v, gate, positions, run: int = 0) -> torch.Tensor:
+        oq, ok, ov = ops.rotary_qkv_prep(q, k, v, positions, self.freq, self.mag, self.rot_dims, self.interleaved, self.num_heads, self.key_dim,
+                                         self.value_dim, 1.0, self.key_dim ** -0.5)
+        w = self.decays.unsqueeze(0).expand(oq.shape[0], self.num_heads)      # one decay per head, the same for every token (row stride 0)
+        o = self.memory(oq, ok, w, ov, run)
+        return ops.group_rmsnorm_gate(o, None, self.value_dim, self.eps, gate, "silu", gate_first=False)
+
+
+class TokenShift(_StatePool):
+    """Blends every token's input with the input of the token before it, once per consumer: out[s] = h + (h_prev - h) mu[s].  The
+    last input of a sequence is carried from step to step in its state slot (fp32 [1, width]; zeros before the first token)."""
+
+    def __init__(self, width: int, consumers: int, state_runs: int = 1):
+        super().__init__((1, width), state_runs)
+        self.width, self.consumers = width, consumers
+        self.mu = nn.Parameter(torch.zeros(consumers, width), requires_grad=False)
+
+    def forward(self, h: torch.Tensor, run: int = 0) -> torch.Tensor:
+        ctx = get_context()
+        return ops.token_shift_mix(h, self.mu.data, self.pool(run), ctx.state_slots, ctx.cu_seqlens_q, ctx.context_lens)
+
+
+class WKV(nn.Module):
+    """The time mix of RWKV-6 ("Eagle and Finch: RWKV with Matrix-Valued States and Dynamic Recurrence", Peng et al.): per head a matrix
+    memory S [dim, dim] in fp32 with a data-dependent decay per key channel, read BEFORE the token is written, the token itself
+    entering its own read-out through a bonus u per head and channel:
+
+        w = exp(-exp(W2 tanh(l) + w0)),      o = (S + diag(u) k v^T)^T r,      S <- diag(w) S + k v^T
+
+    l: a low-rank projection of the (token-shifted) input.  The read-out of a head is divided by its root mean square, multiplied by a
+    weight per column and by silu(gate).
+
+    forward takes r, k, v, gate (projection outputs, each possibly of an input of its own) and the low-rank decay input l."""
+
+    def __init__(self, num_heads: int, head_dim: int, rank: int, eps: float, state_runs: int = 1):
+        super().__init__()
+        n = num_heads * head_dim
+        self.num_heads, self.head_dim, self.rank, self.eps = num_heads, head_dim, rank, eps
+        self.decay_up = MergedLinear(rank, [n], bias=True)                 # W2 and w0
+        self.bonus = nn.Parameter(torch.zeros(num_heads, head_dim, dtype=torch.float32), requires_grad=False)      # (an operand of the fp32 scan)
+        self.norm = nn.Parameter(torch.ones(n), requires_grad=False)
+        self.memory = DiagonalDecayRecurrence(num_heads, head_dim, head_dim, state_runs=state_runs)
+
+    def forward(self, r, k, v, gate, lowrank, run: int = 0) -> torch.Tensor:
+        z = self.decay_up(ops.act_mul(lowrank, "tanh", False), out_f32=True)
+        oq, ok, ow, ov = ops.gla_prep(r, k, v, z, 1.0, decay="exp_exp")
+        o = self.memory(oq, ok, ow, ov, run, read_first=True, bonus=self.bonus.data)
+        return ops.group_rmsnorm_gate(o, self.norm.data, self.head_dim, self.eps, gate, "silu", gate_first=False)

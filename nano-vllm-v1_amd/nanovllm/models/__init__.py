@@ -20,6 +20,8 @@ _REGISTRY = {
     "LamutarForCausalLM": ("lamutar", "LamutarForCausalLM"),
     "Dinatar": ("dinatar", "DinatarForCausalLM"),
     "DinatarForCausalLM": ("dinatar", "DinatarForCausalLM"),
+    "Lakatar": ("lakatar", "LakatarForCausalLM"),
+    "LakatarForCausalLM": ("lakatar", "LakatarForCausalLM"),
 }
 
 

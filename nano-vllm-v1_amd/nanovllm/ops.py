@@ -733,7 +733,7 @@ def delta_post(o: torch.Tensor, norm_weight: torch.Tensor, gate: torch.Tensor | 
 
 # ---------------------------------------------------------------- layer norm / RMS norm around the fp32 stream, plain activations
 NORM_KINDS = {None: 0, "layer": 1, "rms": 2}
-ACTS = {"silu": 0, "gelu_tanh": 1, "relu2": 2}
+ACTS = {"silu": 0, "gelu_tanh": 1, "relu2": 2, "tanh": 3}
 
 
 def embedding_pos_stream(ids: torch.Tensor, positions: torch.Tensor, table: torch.Tensor, pos_table: torch.Tensor | None, scale: float = 1.0) -> torch.Tensor:
@@ -769,8 +769,26 @@ def residual_norm(x: torch.Tensor, a=None, a_weight=None, b=None, b_weight=None,
     return h
 
 
+def residual_postnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, y=None, y32=None, layer_scale=None, alpha: float = 1.0,
+                      weight_offset: float = 0.0, want_h: bool = True, in_place: bool = True) -> torch.Tensor | None:
+    """x <- rms_norm(alpha x + layer_scale (y + y32)) * (weight_offset + weight) in place (fp32 rows; y of the activation type and
+    y32 fp32 may each be absent); returns the new x in the activation type (the input of the next sublayer).  `in_place` False:
+    x is only read."""
+    assert x.dtype == F32 and x.is_contiguous() and x.dim() == 2
+    rows, dim = x.shape
+    typed = [t for t in (weight, y, layer_scale) if t is not None]
+    f = _act_flag(*typed)
+    assert weight.numel() == dim and weight.is_contiguous() and (layer_scale is None or (layer_scale.numel() == dim and layer_scale.is_contiguous()))
+    assert y is None or (y.shape == (rows, dim) and y.stride(1) == 1)
+    assert y32 is None or (y32.dtype == F32 and y32.shape == (rows, dim) and y32.stride(1) == 1)
+    h = torch.empty(rows, dim, dtype=weight.dtype, device=x.device) if want_h else None
+    _hip.call("nvh_residual_postnorm", _p(y), y.stride(0) if y is not None else 0, _p(y32), y32.stride(0) if y32 is not None else 0, _p(layer_scale),
+              float(alpha), x.data_ptr(), int(in_place), weight.data_ptr(), float(weight_offset), float(eps), _p(h), dim, rows, dim, f, _stream())
+    return h
+
+
 def act_mul(x: torch.Tensor, act: str, gated: bool) -> torch.Tensor:
-    """act(x) for plain rows, act(x[:, :I]) * x[:, I:] for a merged [gate | up] projection; act: silu, gelu_tanh, relu2."""
+    """act(x) for plain rows, act(x[:, :I]) * x[:, I:] for a merged [gate | up] projection; act: silu, gelu_tanh, relu2, tanh."""
     f = _act_flag(x)
     assert x.dim() == 2 and x.stride(1) == 1
     rows, inter = x.shape[0], x.shape[1] // 2 if gated else x.shape[1]
@@ -799,11 +817,12 @@ SCAN_SEGMENT_MAX_BATCH = 8         # ... in steps of at most this many sequences
 
 
 def gated_linear_scan(q, k, w, v, state, slots, cu_seqlens_q, context_lens, heads: int, dk: int, dv: int, qk_groups: int | None = None,
-                      kscale=None, skip=None, max_seqlen_q: int = 0) -> torch.Tensor:
+                      kscale=None, skip=None, max_seqlen_q: int = 0, read_first: bool = False, bonus=None) -> torch.Tensor:
     """S <- diag(w) S + (kscale k) v^T, o = S^T q + skip v over the packed tokens; fp32 operands q, k [T, qk_groups * dk],
     w [T, H * dk] or [T, H] (one decay per head), kscale [T, H] | None, v [T, H * dv], skip [H] | None; `state`
     [slots, H, dv, dk] fp32 (S transposed: a column's rows lie together) is read (unless the sequence starts in this step) and
-    left updated.  Returns fp32 [T, H * dv]."""
+    left updated.  Returns fp32 [T, H * dv].  `read_first`: o = (S + diag(bonus) (kscale k) v^T)^T q + skip v is taken BEFORE the
+    token is written and the state decayed (bonus fp32 [H, dk] | None)."""
     t = v.shape[0]
     g = qk_groups or heads
     _f32_rows(t, q, k, w, v)
@@ -811,6 +830,7 @@ def gated_linear_scan(q, k, w, v, state, slots, cu_seqlens_q, context_lens, head
     w_scalar = w.shape[1] == heads and dk != 1
     assert kscale is None or (kscale.dtype == F32 and kscale.shape == (t, heads) and kscale.stride(1) == 1)
     assert skip is None or (skip.dtype == F32 and skip.numel() == heads and skip.is_contiguous())
+    assert bonus is None or (read_first and bonus.dtype == F32 and bonus.numel() == heads * dk and bonus.is_contiguous() and bonus.is_cuda)
     assert state.dtype == F32 and state.is_contiguous() and tuple(state.shape[1:]) == (heads, dv, dk) and slots.dtype == torch.int32
     assert context_lens.dtype == torch.int32 and (cu_seqlens_q is None or cu_seqlens_q.dtype == torch.int32)
     batch = context_lens.numel()
@@ -827,7 +847,7 @@ def gated_linear_scan(q, k, w, v, state, slots, cu_seqlens_q, context_lens, head
     _hip.call("nvh_gated_linear_scan", q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), g, w.data_ptr(), w.stride(0), int(w_scalar),
               _p(kscale), kscale.stride(0) if kscale is not None else 0, v.data_ptr(), v.stride(0), _p(skip), state.data_ptr(), slots.data_ptr(),
               _p(cu_seqlens_q), context_lens.data_ptr(), out.data_ptr(), batch, heads, dk, dv, segments, SCAN_SEGMENT_MIN_TOKENS, _p(ws_l), _p(ws_d),
-              _stream())
+              int(read_first), _p(bonus), _stream())
     return out
 
 
@@ -843,8 +863,9 @@ def hgrn2_prep(q, f, v, f_bias, lower):
     return oq, ok, ow, ov
 
 
-def gla_prep(q, k, v, decay_logits, q_scale: float, tau: float):
-    """fp32 (q * q_scale, k, sigmoid(decay_logits)^(1/tau), v) from projection columns and fp32 decay logits."""
+def gla_prep(q, k, v, decay_logits, q_scale: float, tau: float = 1.0, decay: str = "sigmoid_pow"):
+    """fp32 (q * q_scale, k, w, v) from projection columns and fp32 decay logits z: w = sigmoid(z)^(1/tau) ("sigmoid_pow") or
+    exp(-exp(z)) ("exp_exp")."""
     fl = _act_flag(q, k, v)
     t, nk, nv = q.shape[0], q.shape[1], v.shape[1]
     assert q.stride(1) == 1 and k.stride(1) == 1 and v.stride(1) == 1 and k.shape == (t, nk)
@@ -852,8 +873,44 @@ def gla_prep(q, k, v, decay_logits, q_scale: float, tau: float):
     oq, ok, ow = (torch.empty(t, nk, dtype=F32, device=q.device) for _ in range(3))
     ov = torch.empty(t, nv, dtype=F32, device=q.device)
     _hip.call("nvh_gla_prep", q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), decay_logits.data_ptr(),
-              decay_logits.stride(0), float(q_scale), float(tau), oq.data_ptr(), ok.data_ptr(), ow.data_ptr(), ov.data_ptr(), t, nk, nv, fl, _stream())
+              decay_logits.stride(0), float(q_scale), float(tau), oq.data_ptr(), ok.data_ptr(), ow.data_ptr(), ov.data_ptr(), t, nk, nv,
+              {"sigmoid_pow": 0, "exp_exp": 1}[decay], fl, _stream())
     return oq, ok, ow, ov
+
+
+def token_shift_mix(h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, slots, cu_seqlens_q, context_lens) -> torch.Tensor:
+    """out[s] = h + (previous token's h - h) * mu[s] for every row s of mu [n, dim]: [n, T, dim] in h's type.  The token before a
+    step's first comes from `state` fp32 [slots, 1, dim] (zeros when the sequence starts in this step), which is then left
+    holding the step's last h of every sequence."""
+    f = _act_flag(h, mu)
+    t, dim = h.shape
+    n = mu.shape[0]
+    assert h.stride(1) == 1 and mu.is_contiguous() and mu.shape[1] == dim
+    assert state.dtype == F32 and state.is_contiguous() and state.numel() == state.shape[0] * dim
+    assert slots.dtype == torch.int32 and context_lens.dtype == torch.int32 and (cu_seqlens_q is None or cu_seqlens_q.dtype == torch.int32)
+    batch = context_lens.numel()
+    out = torch.empty(n, t, dim, dtype=h.dtype, device=h.device)
+    _hip.call("nvh_token_shift_mix", h.data_ptr(), h.stride(0), state.data_ptr(), slots.data_ptr(), _p(cu_seqlens_q), context_lens.data_ptr(), batch,
+              mu.data_ptr(), out.data_ptr(), t, n, dim, f, _stream())
+    _hip.call("nvh_conv_state_update", h.data_ptr(), h.stride(0), state.data_ptr(), slots.data_ptr(), _p(cu_seqlens_q), context_lens.data_ptr(), batch,
+              2, dim, f, _stream())
+    return out
+
+
+def rotary_qkv_prep(q, k, v, positions, freq, mag: float, rot_dims: int, interleaved: bool, heads: int, dim: int, vdim: int,
+                    q_scale: float = 1.0, k_scale: float = 1.0):
+    """fp32 (q, k, v) operands of a recurrence from projection columns, with rotary positions on the first `rot_dims` dimensions of
+    every q / k head (freq fp32 [rot_dims / 2]; pairs interleaved or in halves) and q, k scaled after the rotation."""
+    fl = _act_flag(q, k, v)
+    t = q.shape[0]
+    assert q.stride(1) == 1 and k.stride(1) == 1 and v.stride(1) == 1 and q.shape[1] == heads * dim and k.shape[1] == heads * dim and v.shape[1] == heads * vdim
+    assert positions.dtype == torch.int64 and (rot_dims == 0 or (freq.dtype == F32 and freq.numel() * 2 == rot_dims and freq.is_cuda))
+    oq, ok = (torch.empty(t, heads * dim, dtype=F32, device=q.device) for _ in range(2))
+    ov = torch.empty(t, heads * vdim, dtype=F32, device=q.device)
+    _hip.call("nvh_rotary_qkv_prep", q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), positions.data_ptr(), _p(freq),
+              float(mag), rot_dims, int(interleaved), float(q_scale), float(k_scale), oq.data_ptr(), ok.data_ptr(), ov.data_ptr(), t, heads, dim, vdim,
+              fl, _stream())
+    return oq, ok, ov
 
 
 def ssd_conv_prep(xbc, dt, conv_w, conv_b, dt_bias, a_log, conv_state, slots, cu_seqlens_q, context_lens, heads: int, inner: int, gn: int):
@@ -879,16 +936,19 @@ def ssd_conv_prep(xbc, dt, conv_w, conv_b, dt_bias, a_log, conv_state, slots, cu
     return ox, ob, oc, odt, odecay
 
 
-def group_rmsnorm_gate(o: torch.Tensor, weight: torch.Tensor, group_size: int, eps: float, gate=None, gate_act: str | None = None,
-                       gate_first: bool = False) -> torch.Tensor:
+def group_rmsnorm_gate(o: torch.Tensor, weight: torch.Tensor | None, group_size: int, eps: float, gate=None, gate_act: str | None = None,
+                       gate_first: bool = False, out_dtype=None) -> torch.Tensor:
     """RMS norm of fp32 rows over groups of `group_size` columns, times `weight` ([group_size], shared by the groups, or one per
     column), with an optional gate (columns of the activation type; "sigmoid" or "silu") applied before or after the norm."""
-    f = _act_flag(weight) if gate is None else _act_flag(weight, gate)
+    typed = [t for t in (weight, gate) if t is not None]
+    assert typed or out_dtype is not None, "without a weight and a gate the result's type must be named"
+    f = _act_flag(*typed) if typed else int(out_dtype == F32)
     rows, n = o.shape
-    assert o.dtype == F32 and o.is_contiguous() and n % group_size == 0 and weight.numel() in (group_size, n) and weight.is_contiguous()
+    assert o.dtype == F32 and o.is_contiguous() and n % group_size == 0
+    assert weight is None or (weight.numel() in (group_size, n) and weight.is_contiguous())
     assert gate is None or (gate.shape == (rows, n) and gate.stride(1) == 1 and gate_act in ("sigmoid", "silu"))
-    y = torch.empty(rows, n, dtype=weight.dtype, device=o.device)
-    _hip.call("nvh_group_rmsnorm_gate", o.data_ptr(), weight.data_ptr(), int(weight.numel() == n and n != group_size), _p(gate),
+    y = torch.empty(rows, n, dtype=typed[0].dtype if typed else out_dtype, device=o.device)
+    _hip.call("nvh_group_rmsnorm_gate", o.data_ptr(), _p(weight), int(weight is not None and weight.numel() == n and n != group_size), _p(gate),
               gate.stride(0) if gate is not None else 0, {None: 0, "sigmoid": 1, "silu": 2}[gate_act if gate is not None else None], int(gate_first),
               y.data_ptr(), n, rows, n // group_size, group_size, float(eps), f, _stream())
     return y
@@ -943,14 +1003,89 @@ def linear_grouped(x: torch.Tensor, weight: torch.Tensor, plan: dict, gather: bo
     return y
 
 
-def moe_combine(y: torch.Tensor, plan: dict, weights: torch.Tensor, shared: torch.Tensor | None = None) -> torch.Tensor:
-    """fp32 [T, dim]: every token's weighted sum of its choices' rows of y (in choice order), plus `shared` [T, dim]."""
+def moe_combine(y: torch.Tensor, plan: dict, weights: torch.Tensor, shared: torch.Tensor | None = None, shared_gate: torch.Tensor | None = None) -> torch.Tensor:
+    """fp32 [T, dim]: every token's weighted sum of its choices' rows of y (in choice order), plus `shared` [T, dim], which is
+    multiplied by sigmoid(shared_gate[t]) when a gate logit per token (fp32 [T] or a column view) is given."""
     f = _act_flag(y) if shared is None else _act_flag(y, shared)
     t, top = weights.shape
     dim = y.shape[1]
     assert y.stride(1) == 1 and weights.dtype == F32 and weights.is_contiguous() and y.shape[0] == t * top
     assert shared is None or (shared.shape == (t, dim) and shared.stride(1) == 1)
+    assert shared_gate is None or (shared is not None and shared_gate.dtype == F32 and shared_gate.numel() == t and shared_gate.is_cuda)
     out = torch.empty(t, dim, dtype=F32, device=y.device)
     _hip.call("nvh_moe_combine", y.data_ptr(), y.stride(0), plan["pos_of_pair"].data_ptr(), weights.data_ptr(), _p(shared),
-              shared.stride(0) if shared is not None else 0, out.data_ptr(), t, dim, top, f, _stream())
+              shared.stride(0) if shared is not None else 0, _p(shared_gate), shared_gate.reshape(t, -1).stride(0) if shared_gate is not None else 0,
+              out.data_ptr(), t, dim, top, f, _stream())
     return out
+
+
+def moe_route_scored(x: torch.Tensor, weight: torch.Tensor, top: int, correction: torch.Tensor | None = None, groups: int = 1, keep: int = 1,
+                     scale: float = 1.0, aux: torch.Tensor | None = None, want_scores: bool = False):
+    """Routing by softmax scores over all experts of the fp32 logits x @ weight^T: the `top` experts with the largest score +
+    correction among the `keep` best of `groups` equal groups of neighbouring experts (a group's score: its largest corrected
+    score), weighted by their uncorrected scores times `scale`.  `aux` [n, K]: more rows over the same input, returned as fp32
+    products [T, n].  Returns (ids int32 [T, top], weights fp32 [T, top], aux products | None[, scores fp32 [T, E]])."""
+    typed = [t_ for t_ in (x, weight, correction, aux) if t_ is not None]
+    f = _act_flag(*typed)
+    t, k = x.shape
+    e = weight.shape[0]
+    assert x.stride(1) == 1 and weight.is_contiguous() and weight.shape[1] == k and (correction is None or (correction.numel() == e and correction.is_contiguous()))
+    assert aux is None or (aux.is_contiguous() and aux.dim() == 2 and aux.shape[1] == k)
+    n_aux = 0 if aux is None else aux.shape[0]
+    ids = torch.empty(t, top, dtype=torch.int32, device=x.device)
+    weights = torch.empty(t, top, dtype=F32, device=x.device)
+    aux_out = torch.empty(t, n_aux, dtype=F32, device=x.device) if n_aux else None
+    scores = torch.empty(t, e, dtype=F32, device=x.device) if want_scores else None
+    _hip.call("nvh_moe_route_scored", x.data_ptr(), x.stride(0), weight.data_ptr(), _p(correction), _p(aux), _p(aux_out), n_aux, ids.data_ptr(),
+              weights.data_ptr(), _p(scores), t, e, k, top, int(groups), int(keep), float(scale), f, _stream())
+    return (ids, weights, aux_out, scores) if want_scores else (ids, weights, aux_out)
+
+
+# ---------------------------------------------------------------- attention through a low-rank latent
+def latent_prep(proj, q_rank: int, kv_rank: int, rot_dim: int, heads: int, q_norm, kv_norm, eps: float, positions, freq, mag: float,
+                interleaved: bool, k_cache, v_cache, slot_mapping, gated: bool = True):
+    """(normed query latent [T, q_rank], sigmoid gate fp32 [T, H] | None) from the fused projection rows [dq | dkv | gate]; with caches given
+    (a layer that owns its latent) the normed key/value latent and the rotated shared key part go to the tokens' slots: keys
+    [pages, page, 1, kv_rank + rot_dim], values [pages, 1, kv_rank, page].  Without caches the row is [dq | gate]."""
+    own = k_cache is not None
+    typed = [x for x in (proj, q_norm, kv_norm, k_cache, v_cache) if x is not None]
+    f = _act_flag(*typed)
+    t = proj.shape[0]
+    assert proj.stride(1) == 1 and positions.dtype == torch.int64 and q_norm.numel() == q_rank
+    page = 1
+    if own:
+        assert slot_mapping.dtype == torch.int32 and slot_mapping.numel() == t and kv_norm.numel() == kv_rank
+        assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dim() == 4 and tuple(k_cache.shape[2:]) == (1, kv_rank + rot_dim)
+        assert tuple(v_cache.shape) == (k_cache.shape[0], 1, kv_rank, k_cache.shape[1])
+        assert rot_dim == 0 or (freq.dtype == F32 and freq.numel() * 2 == rot_dim)
+        page = k_cache.shape[1]
+    cq = torch.empty(t, q_rank, dtype=proj.dtype, device=proj.device)
+    gate = torch.empty(t, heads, dtype=F32, device=proj.device) if gated else None
+    _hip.call("nvh_latent_prep", proj.data_ptr(), proj.stride(0), q_rank, kv_rank, rot_dim, heads, int(own), q_norm.data_ptr(), _p(kv_norm), float(eps),
+              positions.data_ptr(), _p(freq), float(mag), int(interleaved), cq.data_ptr(), _p(gate), _p(k_cache), _p(v_cache), _p(slot_mapping), page,
+              t, f, _stream())
+    return cq, gate
+
+
+def linear_heads(x: torch.Tensor, weight: torch.Tensor, x_head_stride: int, out: torch.Tensor | None = None, out_head_stride: int | None = None) -> torch.Tensor:
+    """y[t, h, :] = x[t, h x_head_stride : + K] @ weight[h]^T for every head; weight [H, N, K].  `out` (rows of at least H heads of
+    `out_head_stride` elements; default a new [T, H * N]) receives head h's N results at column h * out_head_stride."""
+    f = _act_flag(x, weight)
+    heads, n, k = weight.shape
+    t = x.shape[0]
+    assert weight.is_contiguous() and x.dim() == 2 and x.stride(1) == 1 and x.shape[1] >= (heads - 1) * x_head_stride + k
+    if out is None:
+        out, out_head_stride = torch.empty(t, heads * n, dtype=x.dtype, device=x.device), n
+    assert out.dtype == x.dtype and out.stride(1) == 1 and out.shape[0] == t and out.shape[1] >= (heads - 1) * out_head_stride + n
+    _hip.call("nvh_gemm_heads_nt", x.data_ptr(), x.stride(0), x_head_stride, weight.data_ptr(), out.data_ptr(), out.stride(0), out_head_stride, t, heads, n, k,
+              f, _stream())
+    return out
+
+
+def latent_q_rotary(q: torch.Tensor, positions, freq, mag: float, interleaved: bool, out: torch.Tensor, heads: int, dim: int, rot_dim: int,
+                    out_head: int, out_offset: int) -> None:
+    """out[t, h, out_offset + d] = rotary(q[t, h, dim + d]) for d < rot_dim; q rows [H, dim + rot_dim], out rows [H, out_head]."""
+    f = _act_flag(q, out)
+    assert q.stride(1) == 1 and out.stride(1) == 1 and positions.dtype == torch.int64 and (rot_dim == 0 or (freq.dtype == F32 and freq.numel() * 2 == rot_dim))
+    _hip.call("nvh_latent_q_rotary", q.data_ptr(), q.stride(0), positions.data_ptr(), _p(freq), float(mag), int(interleaved), out.data_ptr(), out.stride(0),
+              q.shape[0], heads, dim, rot_dim, out_head, out_offset, f, _stream())
