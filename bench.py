@@ -495,10 +495,37 @@ def _dinatar_cfg(z):
             "layers": [{"type": mixers[i % 3][0], "mixer": mixers[i % 3][1], "mlp": moe if i % 2 else dense} for i in range(z["layers"])]}
 
 
+def _lakatar_cfg(z):
+    """RWKV-style time-mix, latent-attention and retention layers in turn (the second latent-attention layer reads the latent the
+    first one cached), every feed-forward a mixture of experts routed by scores within groups, sized like Dinatar's expert layers.
+    The cached row of the latent attention is 192 + 64 = 256 wide: the widest the matrix-core attention takes."""
+    w, hd = z["width"], z["head_dim"]
+    yarn = {"factor": 4.0, "original": 4096, "fast": 16.0, "slow": 2.0}
+    latent = {"heads": z["heads"], "dim": hd, "rot_dim": hd // 2, "vdim": hd, "q_rank": 3 * w // 4, "kv_rank": 192, "scale": (hd + hd // 2) ** -0.5,
+              "rot": {"base": 1e6, "dims": hd // 2, "scaling": yarn}}
+    retention = {"heads": w // 256, "dim": 128, "vdim": 256, "decay": [1.0 - 2.0 ** (-5 - 3 * i / max(w // 256 - 1, 1)) for i in range(w // 256)],
+                 "rot": {"base": 1e4, "dims": 128}}
+    mixers = [("wkv", {"heads": w // 64, "dim": 64}), ("latent_attention", latent), ("retention", retention)]
+    moe = {"kind": "moe", "expert": {"ff": z["ff"] // 8}, "router": {"experts": 16, "top": 2, "scale": 1.0, "groups": {"count": 4, "keep": 2}},
+           "shared": {"ff": z["ff"] // 4}}
+    layers, first_latent = [], None
+    for i in range(z["layers"]):
+        kind, mixer = mixers[i % 3]
+        mixer = dict(mixer)
+        if kind == "latent_attention":
+            if first_latent is None:
+                first_latent = i
+            elif "kv_from" not in layers[first_latent]["mixer"] and sum(l["type"] == kind for l in layers) == 1:
+                mixer["kv_from"] = first_latent
+        layers.append({"type": kind, "mixer": mixer, "mlp": moe})
+    return {"architecture": "Lakatar", "vocab": z["vocab"], "width": w, "norm": {"eps": 1e-6}, "postln_alpha": 2.0, "layers": layers}
+
+
 HYBRID_DESIGNS = {
     # --hybrid-design: (the design, the closest model the engine already serves)
     "lamutar": (("lamutar", _lamutar_cfg), ("qwen3", _qwen3_cfg)),
     "dinatar": (("dinatar", _dinatar_cfg), ("lamutar", _lamutar_cfg)),
+    "lakatar": (("lakatar", _lakatar_cfg), ("dinatar", _dinatar_cfg)),
 }
 
 
@@ -506,7 +533,8 @@ def hybrid_compare(args):
     """--hybrid-compare: prefill and decode throughput of a hybrid design (--hybrid-design; operator modules over an fp32 residual
     stream + captured decode graphs) beside the closest model the engine serves at equal width, heads, feed-forward size, depth and
     vocabulary: Lamutar (delta-rule and attention layers in turn) beside Qwen3 (native executor), or Dinatar (windowed attention +
-    Mamba-2, HGRN2, gated linear attention; dense and expert feed-forwards) beside Lamutar.  Random weights, bf16.  One JSON line."""
+    Mamba-2, HGRN2, gated linear attention; dense and expert feed-forwards) beside Lamutar, or Lakatar (RWKV-style time mix, latent
+    attention, retention; score-routed experts; norms after the sums) beside Dinatar.  Random weights, bf16.  One JSON line."""
     import tempfile
     from nanovllm.config import Config
     from nanovllm.engine.model_runner import ModelRunner
