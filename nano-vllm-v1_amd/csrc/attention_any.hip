@@ -145,6 +145,7 @@ struct AttnArgs {
     int window, keep_first;    // window > 0: key j is visible to query i only when i - j < window or j < keep_first
     int pages_offset;          // byte offset in LDS of the sequence's page ids (matrix-core kernel)
     int ml_offset;             // ... and of the waves' (max, sum) pairs in the one-query form
+    int kv_split;              // one-query form: workgroups per (sequence, KV head), each with H / (G kv_split) of the group's heads
 };
 
 // The key tiles (of `tile` keys, starting at multiples of it) that a workgroup whose first query sits at position qlo has to
@@ -338,9 +339,10 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
     }
     if (seq < 0) return;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, fr = lane & 15, fq = lane >> 4;
-    const int group = a.H / a.G;
-    const int kvh = GROUPED ? blockIdx.y : blockIdx.y / group;
-    const int head = GROUPED ? kvh * group + min(fr, group - 1) : blockIdx.y;       // (GROUPED: this lane's row is a head)
+    // GROUPED: blockIdx.y counts (KV head, part of its group of heads); the parts of one KV head read the same keys and values
+    const int group = GROUPED ? a.H / (a.G * a.kv_split) : a.H / a.G;
+    const int kvh = GROUPED ? blockIdx.y / a.kv_split : blockIdx.y / group;
+    const int head = GROUPED ? blockIdx.y * group + min(fr, group - 1) : blockIdx.y;       // (GROUPED: this lane's row is a head)
     const int dim = a.dim, vdim = a.vdim, nks = dim >> 4, nvt = vdim >> 4;
     const int klen = a.context_lens[seq], past = klen - qlen;
     const int nq = GROUPED ? 1 : min(ROWS_Q, qlen - q0);
@@ -359,7 +361,7 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
         for (int i = tid; i < nrows * vdim; i += 256) {
             const int r = i / vdim;
             const int64_t tok = GROUPED ? qbase : qbase + q0 + r;
-            const int hd = GROUPED ? kvh * group + r : (int)blockIdx.y;
+            const int hd = GROUPED ? (int)blockIdx.y * group + r : (int)blockIdx.y;
             ((bf16*)a.out)[(tok * a.H + hd) * vdim + (i - r * vdim)] = (bf16)0.f;
         }
         return;
@@ -551,7 +553,7 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
         const int r = i / half, pair = i - r * half;
         const int c1 = a.v_interleaved ? 2 * pair : pair, c2 = a.v_interleaved ? 2 * pair + 1 : pair + half;
         const int64_t tok = GROUPED ? qbase : qbase + q0 + r;
-        const int hd = GROUPED ? kvh * group + r : (int)blockIdx.y;
+        const int hd = GROUPED ? (int)blockIdx.y * group + r : (int)blockIdx.y;
         float u = os[r * vdim + c1], v = os[r * vdim + c2];
         if (a.v_freq) {
             float sn, cs;
@@ -576,8 +578,15 @@ static void launch_attn_mfma(const AttnArgs& a, int64_t total_q, hipStream_t st)
     b.ml_offset = (int)((b.pages_offset + sizeof(int) * (size_t)a.table_stride + 15) & ~(size_t)15);
     const size_t lds = b.ml_offset + sizeof(float) * 4 * 16 * 2;
     const int group = a.H / a.G;
-    if (total_q == a.batch && group <= 16 && !nvh_switch_on(SW_EXP_A)) {      // one query per sequence: the heads of a KV group share a workgroup
-        attn_paged_mfma_kernel<NKS, NVT, EXACT, 1><<<dim3((unsigned)a.batch, (unsigned)a.G), 256, lds, st>>>(b);
+    // One query per sequence: the heads of a KV group share a workgroup - up to 16 of them; a larger group is cut into parts, and so
+    // is any group while the launch would leave most of the chip idle (the parts of a group then read the same keys and values at
+    // about the same time).  Which part a head falls into does not enter its result.
+    int split = 1;
+    while (group / split > 16 && group % (2 * split) == 0) split *= 2;
+    while ((int64_t)a.batch * a.G * split < 256 && group % (2 * split) == 0 && group / split > 2) split *= 2;
+    if (total_q == a.batch && group / split <= 16 && !nvh_switch_on(SW_EXP_A)) {
+        b.kv_split = split;
+        attn_paged_mfma_kernel<NKS, NVT, EXACT, 1><<<dim3((unsigned)a.batch, (unsigned)(a.G * split)), 256, lds, st>>>(b);
     } else {
         const dim3 grid((unsigned)(total_q / MQ + a.batch), (unsigned)a.H);
         attn_paged_mfma_kernel<NKS, NVT, EXACT, 0><<<grid, 256, lds, st>>>(b);
@@ -585,7 +594,7 @@ static void launch_attn_mfma(const AttnArgs& a, int64_t total_q, hipStream_t st)
 }
 
 // Exact instantiations for the head sizes in use (dim/16, vdim/16); any other 16-aligned pair takes a bounded one.
-#define NVH_ATTN_EXACT(X) X(1, 1) X(2, 2) X(3, 3) X(4, 4) X(5, 5) X(6, 6) X(8, 8) X(12, 12) X(16, 16) X(2, 4) X(4, 2) X(4, 8) X(8, 4) X(8, 16) X(16, 8) X(12, 8)
+#define NVH_ATTN_EXACT(X) X(1, 1) X(2, 2) X(3, 3) X(4, 4) X(5, 5) X(6, 6) X(8, 8) X(12, 12) X(16, 16) X(2, 4) X(4, 2) X(4, 8) X(8, 4) X(8, 16) X(16, 8) X(12, 8) X(16, 12)
 static void dispatch_attn_mfma(const AttnArgs& a, int64_t total_q, hipStream_t st) {
     const int nks = a.dim / 16, nvt = a.vdim / 16;
 #define NVH_ATTN_CASE(K, V)                              \
@@ -645,7 +654,7 @@ extern "C" int32_t nvh_attn_paged_any(const void* q, const void* k_cache, const 
     }
     if (batch == 0 || total_q == 0) return NVH_OK;
     AttnArgs a{q, k_cache, v_cache, cu_seqlens_q, context_lens, block_tables, table_stride, (int)batch, (int)page, (int)num_q_heads,
-               (int)num_kv_heads, (int)dim, (int)vdim, scale, gate, v_freq, v_interleaved, out, slopes, (int)window, (int)keep_first, 0, 0};
+               (int)num_kv_heads, (int)dim, (int)vdim, scale, gate, v_freq, v_interleaved, out, slopes, (int)window, (int)keep_first, 0, 0, 1};
     // at most ceil(len / AQ) tiles per sequence: total_q / AQ + batch bounds their number (surplus workgroups exit)
     const dim3 grid((unsigned)(total_q / AQ + batch), (unsigned)num_q_heads);
     hipStream_t st = (hipStream_t)stream;

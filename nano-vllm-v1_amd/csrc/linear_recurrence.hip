@@ -98,7 +98,7 @@ struct ShiftArgs {
     const void* mu;            // [n, D]
     void* out;                 // [n, T, D]
     int64_t tokens;
-    int n, D;
+    int n, D, vec;
 };
 
 template <typename A>
@@ -112,6 +112,41 @@ __global__ __launch_bounds__(256) void token_shift_mix_kernel(ShiftArgs p) {
     const A* cur = (const A*)p.h + t * p.h_stride;
     const A* prev = first ? nullptr : cur - p.h_stride;
     const float* st = first && carried ? p.state + (int64_t)slot * p.D : nullptr;
+    if (p.vec) {                                             // eight consecutive columns per lane, 16-byte accesses
+        for (int i = threadIdx.x * 8; i < p.D; i += 256 * 8) {
+            float c[8], b[8];
+            nvh_load8(cur, i, 8, true, c);
+            if (prev) {
+                nvh_load8(prev, i, 8, true, b);
+            } else if (st) {
+                nvh_load8(st, i, 8, true, b);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) b[e] = 0.f;
+            }
+            for (int s = 0; s < p.n; ++s) {
+                float m[8];
+                nvh_load8((const A*)p.mu, (int64_t)s * p.D + i, 8, true, m);
+                A* dst = (A*)p.out + ((int64_t)s * p.tokens + t) * p.D + i;
+                if constexpr (sizeof(A) == 2) {
+                    bf16x8 o;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) o[e] = (bf16)(c[e] + (b[e] - c[e]) * m[e]);
+                    *reinterpret_cast<bf16x8*>(dst) = o;
+                } else {
+                    f32x4 lo4, hi4;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        lo4[e] = c[e] + (b[e] - c[e]) * m[e];
+                        hi4[e] = c[4 + e] + (b[4 + e] - c[4 + e]) * m[4 + e];
+                    }
+                    *reinterpret_cast<f32x4*>(dst) = lo4;
+                    *reinterpret_cast<f32x4*>(dst + 4) = hi4;
+                }
+            }
+        }
+        return;
+    }
     for (int i = threadIdx.x; i < p.D; i += 256) {
         const float c = (float)cur[i];
         const float b = prev ? (float)prev[i] : (st ? st[i] : 0.f);
@@ -665,7 +700,8 @@ extern "C" int32_t nvh_token_shift_mix(const void* h, int64_t h_stride, const fl
     NVH_REQUIRE(batch >= 0 && num_tokens >= 0 && num_mixes > 0 && dim > 0 && h_stride >= dim && (cu_seqlens_q || num_tokens == batch), NVH_EINVAL,
                 "nvh_token_shift_mix: bad sizes");
     if (num_tokens == 0 || batch == 0) return NVH_OK;
-    const ShiftArgs p{h, h_stride, state, slots, cu_seqlens_q, context_lens, (int)batch, mu, out, num_tokens, (int)num_mixes, (int)dim};
+    const ShiftArgs p{h, h_stride, state, slots, cu_seqlens_q, context_lens, (int)batch, mu, out, num_tokens, (int)num_mixes, (int)dim,
+                      (int)(dim % 8 == 0 && h_stride % 8 == 0 && nvh_aligned16(h) && nvh_aligned16(state) && nvh_aligned16(mu) && nvh_aligned16(out))};
     hipStream_t st = (hipStream_t)stream;
     if (act_f32) token_shift_mix_kernel<float><<<dim3((unsigned)num_tokens), 256, 0, st>>>(p);
     else token_shift_mix_kernel<bf16><<<dim3((unsigned)num_tokens), 256, 0, st>>>(p);

@@ -161,9 +161,11 @@ __global__ __launch_bounds__(256) void moe_route_scored_kernel(const A* __restri
     const int64_t t = blockIdx.x;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const A* xr = x + t * ldx;
-    constexpr int EG = 4;
+    // every wave takes `eg` rows at a time (up to EG: 17 rows are one pass of five a wave, not two passes of four)
+    constexpr int EG = 8;
     const int rows = experts + n_aux;
-    for (int e0 = wave * EG; e0 < rows; e0 += 4 * EG) {
+    const int eg = min(EG, (rows + 3) / 4);
+    for (int e0 = wave * eg; e0 < rows; e0 += 4 * eg) {
         float acc[EG];
 #pragma unroll
         for (int g = 0; g < EG; ++g) acc[g] = 0.f;
@@ -171,22 +173,24 @@ __global__ __launch_bounds__(256) void moe_route_scored_kernel(const A* __restri
             float xv[8];
             nvh_load8(xr, k0, K - k0, vec, xv);
 #pragma unroll
-            for (int g = 0; g < EG; ++g) {
-                const int e = min(e0 + g, rows - 1);
-                const A* wr = e < experts ? w + (int64_t)e * K : aux + (int64_t)(e - experts) * K;
-                float wv[8];
-                nvh_load8(wr, k0, K - k0, vec, wv);
+            for (int g = 0; g < EG; ++g)
+                if (g < eg) {                                // (uniform)
+                    const int e = min(e0 + g, rows - 1);
+                    const A* wr = e < experts ? w + (int64_t)e * K : aux + (int64_t)(e - experts) * K;
+                    float wv[8];
+                    nvh_load8(wr, k0, K - k0, vec, wv);
 #pragma unroll
-                for (int i = 0; i < 8; ++i) acc[g] = __builtin_fmaf(xv[i], wv[i], acc[g]);
+                    for (int i = 0; i < 8; ++i) acc[g] = __builtin_fmaf(xv[i], wv[i], acc[g]);
+                }
+        }
+#pragma unroll
+        for (int g = 0; g < EG; ++g)
+            if (g < eg) {
+                const int e = e0 + g;
+                const float sum = wave_sum(acc[g]);
+                if (lane == 0 && e < experts) zs[e] = sum;
+                else if (lane == 0 && e < rows) aux_out[t * n_aux + (e - experts)] = sum;
             }
-        }
-#pragma unroll
-        for (int g = 0; g < EG; ++g) {
-            const int e = e0 + g;
-            const float sum = wave_sum(acc[g]);
-            if (lane == 0 && e < experts) zs[e] = sum;
-            else if (lane == 0 && e < rows) aux_out[t * n_aux + (e - experts)] = sum;
-        }
     }
     __syncthreads();
     const bool picker = wave == 0;                           // the first wave picks; the others only keep the barriers company
