@@ -539,7 +539,11 @@ int32_t nvh_attn_paged_any(const void* q, const void* k_cache, const void* v_cac
                            const int32_t* context_lens, const int32_t* block_tables, int64_t table_stride, int64_t batch,
                            int64_t total_q, int64_t page, int64_t num_q_heads, int64_t num_kv_heads, int64_t dim, int64_t vdim,
                            float scale, const float* gate, const float* v_freq, int32_t v_interleaved, const float* slopes,
-                           int64_t window, int64_t keep_first, void* out, int32_t act_f32, nvh_stream_t stream);
+                           int64_t window, int64_t keep_first, void* out, float* parts_ws, int64_t parts_ws_bytes, int32_t act_f32, nvh_stream_t stream);
+/* Bytes of fp32 scratch (parts_ws) with which nvh_attn_paged_any spreads the key tiles of one-query steps over several workgroups
+ * when the launch would otherwise leave most of the chip idle (0: none wanted; without scratch the launch is the plain one). */
+int64_t nvh_attn_paged_any_parts_bytes(int64_t batch, int64_t total_q, int64_t num_q_heads, int64_t num_kv_heads, int64_t dim, int64_t vdim,
+                                       int64_t page, int32_t turned_back, int32_t act_f32);
 
 /* Generalized delta rule, state [slots, H, dk, dv] fp32:  S <- diag(w) S - (a u)(u^T S) + k v^T,  o = S^T r.
  * nvh_delta_prep: out fp32 [T, H, 6, dk] = r | k | w | u | a u | v per head, with w = exp(-decay_scale sigmoid(w0 + w2 tanh(lowrank))),

@@ -146,6 +146,8 @@ struct AttnArgs {
     int pages_offset;          // byte offset in LDS of the sequence's page ids (matrix-core kernel)
     int ml_offset;             // ... and of the waves' (max, sum) pairs in the one-query form
     int kv_split;              // one-query form: workgroups per (sequence, KV head), each with H / (G kv_split) of the group's heads
+    int key_parts;             // one-query form: workgroups that share a sequence's key tiles (tile j goes to part j % key_parts); > 1: the
+    float* parts;              // parts leave [batch, G kv_split, key_parts, 16, vdim + 2] (unnormalised rows, then max and sum) here
 };
 
 // The key tiles (of `tile` keys, starting at multiples of it) that a workgroup whose first query sits at position qlo has to
@@ -357,6 +359,16 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
     constexpr int NKT = SPLIT ? 1 : 4;                       // 16-key blocks of a tile per wave
     const int qpos = GROUPED ? past : past + q0 + qrow;
     const int last_key = past + q0 + nq - 1;
+    const int part = GROUPED ? (int)blockIdx.z : 0, nparts = GROUPED ? a.key_parts : 1;
+    float* prow = nullptr;                                   // this workgroup's record among the parts
+    if (GROUPED && nparts > 1) prow = a.parts + (((int64_t)seq * gridDim.y + blockIdx.y) * nparts + part) * 16 * (vdim + 2);
+    if (last_key < 0 && prow) {                              // a padded row: every part records "no keys", the merge then writes zeros
+        if (tid < 16) {
+            prow[tid * (vdim + 2) + vdim] = -INFINITY;
+            prow[tid * (vdim + 2) + vdim + 1] = 0.f;
+        }
+        return;
+    }
     if (last_key < 0) {                                      // a padded row of a captured step (no keys): zeros, and no address is formed
         for (int i = tid; i < nrows * vdim; i += 256) {
             const int r = i / vdim;
@@ -409,8 +421,18 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
     const float slope = a.slopes ? a.slopes[head] : 0.f;
     const TileWalk walk(a.window, a.keep_first, GROUPED ? past : past + q0, MK);
     bf16x8 kA[KCH], vA[VCH], kB[KCH], vB[VCH];
-    int ka = walk.first_end > 0 || walk.win_start == 0 ? 0 : walk.win_start, kb = walk.next(ka);
-    fetch(ka, kA, vA);
+    // (with key parts a workgroup walks the tiles whose number is its own modulo the number of parts)
+    auto mine = [&](int k0) { return nparts == 1 || (k0 / MK) % nparts == part; };
+    auto next_tile = [&](int k0) {
+        int n = walk.next(k0);
+        while (n <= last_key && !mine(n)) n = walk.next(n);
+        return n;
+    };
+    int ka = walk.first_end > 0 || walk.win_start == 0 ? 0 : walk.win_start;
+    if (!mine(ka)) ka = next_tile(ka);
+    int kb = next_tile(ka);
+    if (ka > last_key) kb = ka;
+    if (ka <= last_key) fetch(ka, kA, vA);
     if (kb <= last_key) fetch(kb, kB, vB);
     auto tile = [&](int k0, int k_after, bf16x8 (&kpre)[KCH], bf16x8 (&vpre)[VCH]) {
         __syncthreads();
@@ -499,10 +521,10 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
             }
     };
     while (ka <= last_key) {
-        const int ka2 = walk.next(kb);
+        const int ka2 = next_tile(kb);
         tile(ka, ka2, kA, vA);
         if (kb > last_key) break;
-        const int kb2 = walk.next(ka2);
+        const int kb2 = next_tile(ka2);
         tile(kb, kb2, kB, vB);
         ka = ka2;
         kb = kb2;
@@ -536,8 +558,17 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
                 num += os[(w * 16 + r) * vdim + col] * f;
                 den += ml[(w * 16 + r) * 2 + 1] * f;
             }
-            os[i] = den > 0.f ? num / den : 0.f;             // (element i of the first wave's rows: read above by this lane only)
+            if (prow) {                                      // a part's record: the row relative to its maximum, then maximum and sum
+                prow[r * (vdim + 2) + col] = num;
+                if (col == 0) {
+                    prow[r * (vdim + 2) + vdim] = big;
+                    prow[r * (vdim + 2) + vdim + 1] = den;
+                }
+            } else {
+                os[i] = den > 0.f ? num / den : 0.f;         // (element i of the first wave's rows: read above by this lane only)
+            }
         }
+        if (prow) return;                                    // (uniform) the merge launch finishes the rows
     } else {
         const float inv_l = l_run > 0.f ? 1.0f / l_run : 0.f;
 #pragma unroll
@@ -569,6 +600,55 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
     }
 }
 
+// The rows of the key parts of a (sequence, group of heads) merged: out = gate * sum_p num_p 2^(m_p - m) / sum_p den_p 2^(m_p - m).
+__global__ __launch_bounds__(256) void attn_merge_parts_kernel(const float* __restrict__ parts, int nparts, int rows, int vdim, int H, const float* __restrict__ gate,
+                                                               bf16* __restrict__ out) {
+    // one workgroup per (sequence, group of heads, row): a lane per value column
+    const int seq = blockIdx.x, hg = blockIdx.y, r = blockIdx.z;
+    const float* base = parts + (((int64_t)seq * gridDim.y + hg) * nparts * 16 + r) * (vdim + 2);
+    const int64_t pstride = (int64_t)16 * (vdim + 2);
+    float big = -INFINITY;
+    for (int p = 0; p < nparts; ++p) big = fmaxf(big, base[p * pstride + vdim]);
+    const int hd = hg * rows + r;
+    const float g = gate ? gate[(int64_t)seq * H + hd] : 1.0f;
+    for (int col = threadIdx.x; col < vdim; col += 256) {
+        float num = 0.f, den = 0.f;
+        for (int p = 0; p < nparts; ++p) {
+            const float* pr = base + p * pstride;
+            if (pr[vdim] == -INFINITY) continue;             // a part without keys (its row is not written)
+            const float f = __builtin_amdgcn_exp2f((pr[vdim] - big) * 1.4426950408889634f);
+            num += pr[col] * f;
+            den += pr[vdim + 1] * f;
+        }
+        out[((int64_t)seq * H + hd) * vdim + col] = (bf16)(den > 0.f ? num / den * g : 0.f);
+    }
+}
+
+// One query per sequence: the heads of a KV group share a workgroup - up to 16 of them; a larger group is cut into parts.  A launch
+// that would leave most of the chip idle is widened: where nothing turns the values back (no v_freq) by giving a sequence's key
+// tiles to several workgroups in turn, whose rows a second launch merges (the keys and values are still read once); otherwise by
+// cutting the group of heads further (its parts then read the same keys and values at about the same time).  Which workgroup a
+// head or a tile falls to enters the result within fp32 rounding only (the order of the merge).
+struct OneQueryPlan {
+    int split, key_parts;
+};
+static OneQueryPlan one_query_plan(int64_t batch, int H, int G, bool turned_back) {
+    const int group = H / G;
+    int split = 1;
+    while (group / split > 16 && group % (2 * split) == 0) split *= 2;
+    int parts = 1;
+    if (!turned_back) {
+        while (batch * G * split * parts * 2 <= 256 && parts < 16) parts *= 2;       // (two workgroups a CU measured slower: 53 against 37 us)
+    } else {
+        while (batch * G * split < 256 && group % (2 * split) == 0 && group / split > 2) split *= 2;
+    }
+    return OneQueryPlan{split, parts};
+}
+static size_t one_query_parts_bytes(int64_t batch, int H, int G, int vdim, bool turned_back) {
+    const OneQueryPlan pl = one_query_plan(batch, H, G, turned_back);
+    return pl.key_parts > 1 ? sizeof(float) * (size_t)batch * G * pl.split * pl.key_parts * 16 * (vdim + 2) : 0;
+}
+
 template <int NKS, int NVT, bool EXACT>
 static void launch_attn_mfma(const AttnArgs& a, int64_t total_q, hipStream_t st) {
     const size_t tiles = sizeof(bf16) * ((size_t)MK * (a.dim + 8) + (size_t)a.vdim * (MK + 8));
@@ -578,15 +658,15 @@ static void launch_attn_mfma(const AttnArgs& a, int64_t total_q, hipStream_t st)
     b.ml_offset = (int)((b.pages_offset + sizeof(int) * (size_t)a.table_stride + 15) & ~(size_t)15);
     const size_t lds = b.ml_offset + sizeof(float) * 4 * 16 * 2;
     const int group = a.H / a.G;
-    // One query per sequence: the heads of a KV group share a workgroup - up to 16 of them; a larger group is cut into parts, and so
-    // is any group while the launch would leave most of the chip idle (the parts of a group then read the same keys and values at
-    // about the same time).  Which part a head falls into does not enter its result.
-    int split = 1;
-    while (group / split > 16 && group % (2 * split) == 0) split *= 2;
-    while ((int64_t)a.batch * a.G * split < 256 && group % (2 * split) == 0 && group / split > 2) split *= 2;
-    if (total_q == a.batch && group / split <= 16 && !nvh_switch_on(SW_EXP_A)) {
-        b.kv_split = split;
-        attn_paged_mfma_kernel<NKS, NVT, EXACT, 1><<<dim3((unsigned)a.batch, (unsigned)(a.G * split)), 256, lds, st>>>(b);
+    OneQueryPlan pl = one_query_plan(a.batch, a.H, a.G, a.v_freq != nullptr);
+    if (!a.parts) pl.key_parts = 1;
+    if (total_q == a.batch && group / pl.split <= 16 && !nvh_switch_on(SW_EXP_A)) {
+        b.kv_split = pl.split;
+        b.key_parts = pl.key_parts;
+        attn_paged_mfma_kernel<NKS, NVT, EXACT, 1><<<dim3((unsigned)a.batch, (unsigned)(a.G * pl.split), (unsigned)pl.key_parts), 256, lds, st>>>(b);
+        if (pl.key_parts > 1)
+            attn_merge_parts_kernel<<<dim3((unsigned)a.batch, (unsigned)(a.G * pl.split), (unsigned)(group / pl.split)), 256, 0, st>>>(a.parts, pl.key_parts, group / pl.split, a.vdim, a.H, a.gate,
+                                                                                                        (bf16*)a.out);
     } else {
         const dim3 grid((unsigned)(total_q / MQ + a.batch), (unsigned)a.H);
         attn_paged_mfma_kernel<NKS, NVT, EXACT, 0><<<grid, 256, lds, st>>>(b);
@@ -638,7 +718,8 @@ extern "C" int32_t nvh_attn_paged_any(const void* q, const void* k_cache, const 
                                       const int32_t* context_lens, const int32_t* block_tables, int64_t table_stride, int64_t batch,
                                       int64_t total_q, int64_t page, int64_t num_q_heads, int64_t num_kv_heads, int64_t dim, int64_t vdim,
                                       float scale, const float* gate, const float* v_freq, int32_t v_interleaved, const float* slopes,
-                                      int64_t window, int64_t keep_first, void* out, int32_t act_f32, nvh_stream_t stream) {
+                                      int64_t window, int64_t keep_first, void* out, float* parts_ws, int64_t parts_ws_bytes, int32_t act_f32,
+                                      nvh_stream_t stream) {
     NVH_REQUIRE(window >= 0 && keep_first >= 0 && window < (1 << 30) && keep_first < (1 << 30), NVH_EINVAL, "nvh_attn_paged_any: bad window");
     NVH_REQUIRE(q && k_cache && v_cache && context_lens && block_tables && out, NVH_EINVAL, "nvh_attn_paged_any: null pointer");
     NVH_REQUIRE(batch >= 0 && total_q >= 0 && page > 0 && num_q_heads > 0 && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0 && dim > 0 && vdim > 0,
@@ -654,7 +735,7 @@ extern "C" int32_t nvh_attn_paged_any(const void* q, const void* k_cache, const 
     }
     if (batch == 0 || total_q == 0) return NVH_OK;
     AttnArgs a{q, k_cache, v_cache, cu_seqlens_q, context_lens, block_tables, table_stride, (int)batch, (int)page, (int)num_q_heads,
-               (int)num_kv_heads, (int)dim, (int)vdim, scale, gate, v_freq, v_interleaved, out, slopes, (int)window, (int)keep_first, 0, 0, 1};
+               (int)num_kv_heads, (int)dim, (int)vdim, scale, gate, v_freq, v_interleaved, out, slopes, (int)window, (int)keep_first, 0, 0, 1, 1, nullptr};
     // at most ceil(len / AQ) tiles per sequence: total_q / AQ + batch bounds their number (surplus workgroups exit)
     const dim3 grid((unsigned)(total_q / AQ + batch), (unsigned)num_q_heads);
     hipStream_t st = (hipStream_t)stream;
@@ -662,6 +743,9 @@ extern "C" int32_t nvh_attn_paged_any(const void* q, const void* k_cache, const 
     const bool mfma = !act_f32 && dim % 16 == 0 && vdim % 16 == 0 && dim <= 256 && vdim <= 256 && page % MK == 0 && nvh_aligned16(q) && nvh_aligned16(k_cache) &&
                       nvh_aligned16(v_cache) && !nvh_switch_on(SW_ATTN_ANY_NO_MFMA);
     if (mfma) {
+        // (scratch for the key parts of the one-query form: used when it is given and large enough, see nvh_attn_paged_any_parts_bytes)
+        const size_t need = total_q == batch ? one_query_parts_bytes(batch, (int)num_q_heads, (int)num_kv_heads, (int)vdim, v_freq != nullptr) : 0;
+        if (parts_ws && need && (size_t)parts_ws_bytes >= need) a.parts = parts_ws;
         dispatch_attn_mfma(a, total_q, st);
     } else if (act_f32) {
         attn_paged_any_kernel<float><<<grid, 256, lds, st>>>(a);
@@ -670,4 +754,11 @@ extern "C" int32_t nvh_attn_paged_any(const void* q, const void* k_cache, const 
     }
     NVH_CHECK_LAUNCH("nvh_attn_paged_any");
     return NVH_OK;
+}
+
+extern "C" int64_t nvh_attn_paged_any_parts_bytes(int64_t batch, int64_t total_q, int64_t num_q_heads, int64_t num_kv_heads, int64_t dim, int64_t vdim,
+                                                  int64_t page, int32_t turned_back, int32_t act_f32) {
+    if (batch <= 0 || total_q != batch || act_f32 || num_kv_heads <= 0 || num_q_heads % num_kv_heads) return 0;
+    if (dim % 16 || vdim % 16 || dim > 256 || vdim > 256 || page % MK) return 0;           // (the matrix-core kernel's sizes)
+    return (int64_t)one_query_parts_bytes(batch, (int)num_q_heads, (int)num_kv_heads, (int)vdim, turned_back != 0);
 }

@@ -150,14 +150,15 @@ __global__ __launch_bounds__(256) void moe_route_linear_kernel(const A* __restri
 // experts are taken (ties: lower id) and weighted by their s times `scale`, not renormalised.  `aux` [n_aux, K]: further
 // rows that read the same input; their fp32 products go to aux_out [T, n_aux] (a gate of the layer, say).
 // One workgroup per token, products as in moe_route_linear_kernel; the first wave picks.
-template <typename A>
+// PL: experts (and groups) a lane of the picking wave holds: experts <= 64 PL.
+template <typename A, int PL>
 __global__ __launch_bounds__(256) void moe_route_scored_kernel(const A* __restrict__ x, int64_t ldx, const A* __restrict__ w, const A* __restrict__ correction,
                                                                const A* __restrict__ aux, float* __restrict__ aux_out, int n_aux, int32_t* __restrict__ ids,
                                                                float* __restrict__ weights, float* __restrict__ scores_out, int experts, int K, int top,
                                                                int groups, int keep, float scale, int vec) {
-    __shared__ float zs[64 * ROUTE_MAX_PER_LANE];            // logits, then scores
-    __shared__ float cs[64 * ROUTE_MAX_PER_LANE];            // choice scores
-    __shared__ float gsc[64 * ROUTE_MAX_PER_LANE];           // group scores
+    __shared__ float zs[64 * PL];            // logits, then scores
+    __shared__ float cs[64 * PL];            // choice scores
+    __shared__ float gsc[64 * PL];           // 1 for a kept group
     const int64_t t = blockIdx.x;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const A* xr = x + t * ldx;
@@ -195,24 +196,24 @@ __global__ __launch_bounds__(256) void moe_route_scored_kernel(const A* __restri
     __syncthreads();
     const bool picker = wave == 0;                           // the first wave picks; the others only keep the barriers company
     // softmax over all experts
-    float z[ROUTE_MAX_PER_LANE];
+    float z[PL];
     if (picker) {
         float mx = -INFINITY;
 #pragma unroll
-        for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j) {
+        for (int j = 0; j < PL; ++j) {
             z[j] = lane + 64 * j < experts ? zs[lane + 64 * j] : -INFINITY;
             mx = fmaxf(mx, z[j]);
         }
         mx = wave_max(mx);
         float den = 0.f;
 #pragma unroll
-        for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j) {
+        for (int j = 0; j < PL; ++j) {
             z[j] = lane + 64 * j < experts ? expf(z[j] - mx) : 0.f;
             den += z[j];
         }
         den = wave_sum(den);
 #pragma unroll
-        for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j) {
+        for (int j = 0; j < PL; ++j) {
             const int e = lane + 64 * j;
             if (e < experts) {
                 const float sc = z[j] / den;
@@ -228,11 +229,11 @@ __global__ __launch_bounds__(256) void moe_route_scored_kernel(const A* __restri
     __syncthreads();
     if (groups > 1 && keep < groups) {                       // (uniform)
         const int gsz = experts / groups;
-        float gv[ROUTE_MAX_PER_LANE];
-        bool gone[ROUTE_MAX_PER_LANE];
+        float gv[PL];
+        bool gone[PL];
         if (picker) {
 #pragma unroll
-            for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j) {
+            for (int j = 0; j < PL; ++j) {
                 const int g = lane + 64 * j;
                 gone[j] = g >= groups;
                 gv[j] = -INFINITY;
@@ -248,7 +249,7 @@ __global__ __launch_bounds__(256) void moe_route_scored_kernel(const A* __restri
                 float bv = -INFINITY;
                 int bg = 0x7fffffff;
 #pragma unroll
-                for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j)
+                for (int j = 0; j < PL; ++j)
                     if (!gone[j] && (bg == 0x7fffffff || gv[j] > bv)) {
                         bv = gv[j];
                         bg = lane + 64 * j;
@@ -264,28 +265,28 @@ __global__ __launch_bounds__(256) void moe_route_scored_kernel(const A* __restri
                 }
                 if (lane == 0) gsc[bg] = 1.f;
 #pragma unroll
-                for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j)
+                for (int j = 0; j < PL; ++j)
                     if (lane + 64 * j == bg) gone[j] = true;
             }
         }
         __syncthreads();
         if (picker) {
 #pragma unroll
-            for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j) {
+            for (int j = 0; j < PL; ++j) {
                 const int e = lane + 64 * j;
                 if (e < experts && gsc[e / gsz] == 0.f) z[j] = -INFINITY;
             }
         }
     }
     if (!picker) return;
-    bool taken[ROUTE_MAX_PER_LANE];
+    bool taken[PL];
 #pragma unroll
-    for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j) taken[j] = lane + 64 * j >= experts;
+    for (int j = 0; j < PL; ++j) taken[j] = lane + 64 * j >= experts;
     for (int r = 0; r < top; ++r) {
         float bv = -INFINITY;
         int be = 0x7fffffff;
 #pragma unroll
-        for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j) {
+        for (int j = 0; j < PL; ++j) {
             const int e = lane + 64 * j;
             if (!taken[j] && (z[j] > bv || be == 0x7fffffff)) {
                 bv = z[j];
@@ -306,7 +307,7 @@ __global__ __launch_bounds__(256) void moe_route_scored_kernel(const A* __restri
             weights[t * top + r] = zs[be] * scale;
         }
 #pragma unroll
-        for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j)
+        for (int j = 0; j < PL; ++j)
             if (lane + 64 * j == be) taken[j] = true;
     }
 }
@@ -448,8 +449,18 @@ extern "C" int32_t nvh_moe_route_scored(const void* x, int64_t x_row_stride, con
     const dim3 grid((unsigned)num_tokens);
     hipStream_t st = (hipStream_t)stream;
     const int vec = K % 8 == 0 && x_row_stride % 8 == 0 && nvh_aligned16(x) && nvh_aligned16(w) && (!aux || nvh_aligned16(aux));
-    if (act_f32) moe_route_scored_kernel<float><<<grid, 256, 0, st>>>((const float*)x, x_row_stride, (const float*)w, (const float*)correction, (const float*)aux, aux_out, (int)num_aux, ids, weights, scores_out, (int)experts, (int)K, (int)top, (int)groups, (int)keep, scale, vec);
-    else moe_route_scored_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)x, x_row_stride, (const bf16*)w, (const bf16*)correction, (const bf16*)aux, aux_out, (int)num_aux, ids, weights, scores_out, (int)experts, (int)K, (int)top, (int)groups, (int)keep, scale, vec);
+#define NVH_ROUTE_SCORED(A, PL) moe_route_scored_kernel<A, PL><<<grid, 256, 0, st>>>((const A*)x, x_row_stride, (const A*)w, (const A*)correction, (const A*)aux, aux_out, (int)num_aux, ids, weights, scores_out, (int)experts, (int)K, (int)top, (int)groups, (int)keep, scale, vec)
+    if (experts <= 64) {
+        if (act_f32) NVH_ROUTE_SCORED(float, 1);
+        else NVH_ROUTE_SCORED(bf16, 1);
+    } else if (experts <= 256) {
+        if (act_f32) NVH_ROUTE_SCORED(float, 4);
+        else NVH_ROUTE_SCORED(bf16, 4);
+    } else {
+        if (act_f32) NVH_ROUTE_SCORED(float, ROUTE_MAX_PER_LANE);
+        else NVH_ROUTE_SCORED(bf16, ROUTE_MAX_PER_LANE);
+    }
+#undef NVH_ROUTE_SCORED
     NVH_CHECK_LAUNCH("nvh_moe_route_scored");
     return NVH_OK;
 }

@@ -98,7 +98,8 @@ SIGNATURES = {
     "nvh_logit_softcap": (i32, [vp, i64, vp, i64, i64, f32, i32, vp]),
     "nvh_gemm_any_nt": (i32, [vp, i64, vp, vp, vp, i64, i64, i64, i64, i32, i32, vp]),
     "nvh_attn_rotary_prep": (i32, [vp, i64, vp, vp, f32, vp, vp, f32, i64, i32, vp, i32, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i32, vp]),
-    "nvh_attn_paged_any": (i32, [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64, f32, vp, vp, i32, vp, i64, i64, vp, i32, vp]),
+    "nvh_attn_paged_any": (i32, [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64, f32, vp, vp, i32, vp, i64, i64, vp, vp, i64, i32, vp]),
+    "nvh_attn_paged_any_parts_bytes": (i64, [i64, i64, i64, i64, i64, i64, i64, i32, i32]),
     "nvh_delta_prep": (i32, [vp, i64, vp, i64, vp, i64, vp, i64, vp, i64, vp, vp, vp, vp, i64, i64, i64, i64, f32, i32, vp]),
     "nvh_delta_scan": (i32, [vp, vp, vp, vp, vp, vp, i64, i64, i64, vp]),
     "nvh_delta_post": (i32, [vp, vp, vp, i64, vp, i64, i64, i64, i64, f32, i32, vp]),

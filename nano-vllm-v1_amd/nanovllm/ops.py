@@ -692,9 +692,12 @@ def attn_paged_any(q, k_cache, v_cache, cu_seqlens_q, context_lens, block_tables
     assert gate is None or (gate.dtype == F32 and gate.shape == (t, heads) and gate.is_contiguous())
     assert slopes is None or (slopes.dtype == F32 and slopes.numel() == heads and slopes.is_contiguous() and slopes.is_cuda)
     out = torch.empty(t, heads * vdim, dtype=q.dtype, device=q.device)
+    # one-query steps that would leave most of the chip idle spread a sequence's key tiles over several workgroups: scratch for their rows
+    ws_bytes = int(_hip.lib().nvh_attn_paged_any_parts_bytes(batch, t, heads, kv_heads, dim, vdim, k_cache.shape[1], int(v_freq is not None), f))
+    ws = torch.empty(ws_bytes // 4, dtype=F32, device=q.device) if ws_bytes else None
     _hip.call("nvh_attn_paged_any", q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _p(cu_seqlens_q), context_lens.data_ptr(),
               block_tables.data_ptr(), block_tables.stride(0), batch, t, k_cache.shape[1], heads, kv_heads, dim, vdim, float(scale),
-              _p(gate), _p(v_freq), int(v_interleaved), _p(slopes), int(window), int(keep_first), out.data_ptr(), f, _stream())
+              _p(gate), _p(v_freq), int(v_interleaved), _p(slopes), int(window), int(keep_first), out.data_ptr(), _p(ws), ws_bytes, f, _stream())
     return out
 
 
