@@ -579,7 +579,7 @@ def main():
     ap.add_argument("--hybrid-compare", action="store_true",
                     help="instead of the headline workload: a hybrid design beside the closest model at equal layer sizes (see hybrid_compare)")
     ap.add_argument("--hybrid-design", default="lamutar", choices=sorted(HYBRID_DESIGNS),
-                    help="lamutar (beside Qwen3; the default) or dinatar (beside Lamutar)")
+                    help="lamutar (beside Qwen3; the default), dinatar (beside Lamutar) or lakatar (beside Dinatar)")
     ap.add_argument("--hybrid-sizes", default="", help="comma-separated subset of " + ",".join(HYBRID_SIZES))
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)

@@ -125,7 +125,7 @@ __global__ __launch_bounds__(256) void attn_rotary_prep_kernel(PrepArgs a) {
 // ---------------------------------------------------------------------------------------------------------------
 constexpr int AQ = 16;        // queries per workgroup (one 16-lane row of a wave per query)
 constexpr int AK = 32;        // keys per tile
-constexpr int AVC = 16;       // value columns per lane: vdim <= 16 * AVC
+constexpr int AVC_MAX = 32;   // value columns per lane (the kernel's AVC: 16, or 32 for wide values): vdim <= 16 * AVC_MAX
 
 struct AttnArgs {
     const void* q;             // [T, H*dim]
@@ -169,7 +169,7 @@ __device__ __forceinline__ bool key_visible(int key, int qpos, int window, int k
     return key <= qpos && (window <= 0 || qpos - key < window || key < keep_first);
 }
 
-template <typename A>
+template <typename A, int AVC>
 __global__ __launch_bounds__(256) void attn_paged_any_kernel(AttnArgs a) {
     extern __shared__ float smem[];
     // which (sequence, query tile) is this workgroup's
@@ -724,14 +724,16 @@ extern "C" int32_t nvh_attn_paged_any(const void* q, const void* k_cache, const 
     NVH_REQUIRE(q && k_cache && v_cache && context_lens && block_tables && out, NVH_EINVAL, "nvh_attn_paged_any: null pointer");
     NVH_REQUIRE(batch >= 0 && total_q >= 0 && page > 0 && num_q_heads > 0 && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0 && dim > 0 && vdim > 0,
                 NVH_EINVAL, "nvh_attn_paged_any: bad sizes");
-    NVH_REQUIRE(vdim <= 16 * AVC, NVH_ENOSYS, "nvh_attn_paged_any: vdim %ld above %d", (long)vdim, 16 * AVC);
+    NVH_REQUIRE(vdim <= 16 * AVC_MAX, NVH_ENOSYS, "nvh_attn_paged_any: vdim %ld above %d", (long)vdim, 16 * AVC_MAX);
     NVH_REQUIRE(!v_freq || vdim % 2 == 0, NVH_EINVAL, "nvh_attn_paged_any: rotated values need an even vdim");
     const size_t lds = sizeof(float) * (size_t)(AQ * dim + AK * (dim + 1) + AK * (vdim + 1) + AQ * AK);
     NVH_REQUIRE(lds <= 160 * 1024, NVH_ENOSYS, "nvh_attn_paged_any: dim %ld + vdim %ld need %zu bytes of LDS", (long)dim, (long)vdim, lds);
     if (lds > 64 * 1024) {                                   // beyond the default limit of dynamic LDS: raise it for both forms (gfx950: 160 KB per workgroup)
-        const hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_paged_any_kernel<float>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        const hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_paged_any_kernel<bf16>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        NVH_REQUIRE(e1 == hipSuccess && e2 == hipSuccess, NVH_ENOSYS, "nvh_attn_paged_any: %zu bytes of LDS refused", lds);
+        const hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_paged_any_kernel<float, 16>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        const hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_paged_any_kernel<bf16, 16>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        const hipError_t e3 = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_paged_any_kernel<float, 32>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        const hipError_t e4 = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_paged_any_kernel<bf16, 32>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        NVH_REQUIRE(e1 == hipSuccess && e2 == hipSuccess && e3 == hipSuccess && e4 == hipSuccess, NVH_ENOSYS, "nvh_attn_paged_any: %zu bytes of LDS refused", lds);
     }
     if (batch == 0 || total_q == 0) return NVH_OK;
     AttnArgs a{q, k_cache, v_cache, cu_seqlens_q, context_lens, block_tables, table_stride, (int)batch, (int)page, (int)num_q_heads,
@@ -747,10 +749,12 @@ extern "C" int32_t nvh_attn_paged_any(const void* q, const void* k_cache, const 
         const size_t need = total_q == batch ? one_query_parts_bytes(batch, (int)num_q_heads, (int)num_kv_heads, (int)vdim, v_freq != nullptr) : 0;
         if (parts_ws && need && (size_t)parts_ws_bytes >= need) a.parts = parts_ws;
         dispatch_attn_mfma(a, total_q, st);
-    } else if (act_f32) {
-        attn_paged_any_kernel<float><<<grid, 256, lds, st>>>(a);
+    } else if (vdim <= 256) {                                // (16 value columns a lane; the choice depends on the size alone)
+        if (act_f32) attn_paged_any_kernel<float, 16><<<grid, 256, lds, st>>>(a);
+        else attn_paged_any_kernel<bf16, 16><<<grid, 256, lds, st>>>(a);
     } else {
-        attn_paged_any_kernel<bf16><<<grid, 256, lds, st>>>(a);
+        if (act_f32) attn_paged_any_kernel<float, 32><<<grid, 256, lds, st>>>(a);
+        else attn_paged_any_kernel<bf16, 32><<<grid, 256, lds, st>>>(a);
     }
     NVH_CHECK_LAUNCH("nvh_attn_paged_any");
     return NVH_OK;
