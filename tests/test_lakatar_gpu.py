@@ -685,3 +685,28 @@ def test_captured_decode_steps_match_eager_ones(flat_case):
         want = flat_case.ref(t)
         for step in range(6):
             assert rel_err(logits[False][step, i:i + 1], want[len(t) - 6 + step:len(t) - 5 + step]) < TOL["float32"]
+
+
+def test_the_replay_program_steps_through_a_schedule(tmp_path, mix_case_calm):
+    """bin/trace_run as a user starts it: steps on standard input, `done <n>` after each, logits of the wanted places in <out>/<n>.f32;
+    a request that is left out of a step and goes on later, one that ends and whose pages and slot the next one takes over."""
+    import subprocess
+    import sys
+    from conftest import ROOT
+    a, b = tokens_of(CFG_MIX, 40, 91), tokens_of(CFG_MIX, 12, 92)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:25], "want": [0, 24]}], "end": []},
+             {"step": 1, "entries": [{"id": "b", "tokens": b[:10], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "a", "tokens": a[25:39], "want": [13]}, {"id": "b", "tokens": b[10:], "want": [1]}], "end": ["b"]},
+             {"step": 3, "entries": [{"id": "a", "tokens": a[39:], "want": [0]}], "end": ["a"]}]
+    for dtype in ("bfloat16", "float32"):
+        out = tmp_path / dtype
+        done = subprocess.run([sys.executable, str(ROOT / "bin" / "trace_run"), "--model", mix_case_calm.path, "--dtype", dtype, "--out", str(out), "--max-tokens", "128"],
+                              input="".join(json.dumps(st) + "\n" for st in steps), capture_output=True, text=True, timeout=600)
+        assert done.returncode == 0, done.stderr[-2000:]
+        assert [ln for ln in done.stdout.splitlines() if ln.startswith("done")] == [f"done {n}" for n in range(4)]
+        assert not (out / "1.f32").exists()
+        ra, rb = mix_case_calm.ref(a), mix_case_calm.ref(b)
+        want = {0: ra[[0, 24]], 2: np.concatenate([ra[38:39], rb[11:12]]), 3: ra[39:40]}
+        for n, w in want.items():
+            got = np.fromfile(out / f"{n}.f32", dtype="<f4").reshape(-1, CFG_MIX["vocab"])
+            assert got.shape == w.shape and rel_err(got, w) < TOL[dtype], (dtype, n)
