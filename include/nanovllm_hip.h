@@ -583,7 +583,7 @@ int32_t nvh_residual_postnorm(const void* y, int64_t y_stride, const float* y32,
                               float* x, int32_t write_x, const void* norm_weight, float weight_offset, float eps, void* h, int64_t h_stride,
                               int64_t rows, int64_t dim, int32_t act_f32, nvh_stream_t stream);
 /* y[rows, inter] = act(x[:, :inter]) (* x[:, inter:2 inter] when gated), evaluated in fp32.  act 0: silu, 1: gelu (tanh form),
- * 2: squared relu, 3: tanh. */
+ * 2: squared relu. */
 int32_t nvh_act_mul(const void* x, int64_t row_stride, void* y, int64_t y_stride, int64_t rows, int64_t inter, int32_t act, int32_t gated,
                     int32_t act_f32, nvh_stream_t stream);
 /* out fp32 [rows, vocab] = scale * logits, softcapped when cap > 0. */
@@ -601,8 +601,7 @@ int32_t nvh_logits_scale(const void* logits, int64_t row_stride, float* out, int
  * read_first: a token is read out before it is written and decayed, o = (S + diag(u) (c k) v^T)^T q + d v, then
  * S <- diag(w) S + (c k) v^T, with the bonus u fp32 [H, dk] (NULL: 0) for the token itself (the RWKV time mix).
  * nvh_hgrn2_prep: q = silu(q), w = f = lower + (1 - lower) sigmoid(f + f_bias), k = 1 - f, v.
- * nvh_gla_prep: q * q_scale, k, v, w = sigmoid(decay_logits)^(1 / tau) (decay_logits fp32; decay_kind 0), or
- * w = exp(-exp(decay_logits)) (decay_kind 1).
+ * nvh_gla_prep: q * q_scale, k, v, w = sigmoid(decay_logits)^(1 / tau) (decay_logits fp32).
  * nvh_token_shift_mix: out[s, t, :] (type A, [num_mixes, T, dim]) = h_t + (h_(t-1) - h_t) mu[s, :], h_(t-1) of a step's
  * first token taken from state fp32 [slots, dim] (zeros at a sequence's start); nvh_conv_state_update with two taps
  * then leaves every sequence's last h in its slot.
@@ -630,8 +629,12 @@ int32_t nvh_hgrn2_prep(const void* q, int64_t q_stride, const void* f, int64_t f
                        int64_t num_tokens, int64_t n_k, int64_t n_v, int32_t act_f32, nvh_stream_t stream);
 int32_t nvh_gla_prep(const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v, int64_t v_stride,
                      const float* decay_logits, int64_t z_stride, float q_scale, float tau, float* out_q, float* out_k,
-                     float* out_w, float* out_v, int64_t num_tokens, int64_t n_k, int64_t n_v, int32_t decay_kind, int32_t act_f32,
-                     nvh_stream_t stream);
+                     float* out_w, float* out_v, int64_t num_tokens, int64_t n_k, int64_t n_v, int32_t act_f32, nvh_stream_t stream);
+/* nvh_wkv_prep: r, k, v -> fp32 operands and the decay w = exp(-exp(w0 + w2 tanh(lowrank))) per key channel (lowrank [T, rank],
+ * w2 [n_k, rank], w0 [n_k], type A; the product in fp32). */
+int32_t nvh_wkv_prep(const void* r, int64_t r_stride, const void* k, int64_t k_stride, const void* v, int64_t v_stride, const void* lowrank,
+                     int64_t lowrank_stride, const void* w2, const void* w0, float* out_q, float* out_k, float* out_w, float* out_v,
+                     int64_t num_tokens, int64_t n_k, int64_t n_v, int64_t rank, int32_t act_f32, nvh_stream_t stream);
 int32_t nvh_token_shift_mix(const void* h, int64_t h_stride, const float* state, const int32_t* slots, const int32_t* cu_seqlens_q,
                             const int32_t* context_lens, int64_t batch, const void* mu, void* out, int64_t num_tokens, int64_t num_mixes,
                             int64_t dim, int32_t act_f32, nvh_stream_t stream);

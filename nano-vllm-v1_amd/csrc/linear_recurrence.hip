@@ -69,7 +69,6 @@ struct GlaPrepArgs {
     float q_scale, inv_tau;
     float *oq, *ok, *ow, *ov;
     int64_t n_k, n_v;
-    int decay_kind;            // 0: sigmoid(z)^(1/tau); 1: exp(-exp(z))
 };
 
 template <typename A>
@@ -78,8 +77,36 @@ __global__ __launch_bounds__(256) void gla_prep_kernel(GlaPrepArgs p) {
     for (int64_t i = threadIdx.x; i < p.n_k; i += 256) {
         p.oq[t * p.n_k + i] = ldf((const A*)p.q, t * p.q_stride + i) * p.q_scale;
         p.ok[t * p.n_k + i] = ldf((const A*)p.k, t * p.k_stride + i);
-        const float z = p.z[t * p.z_stride + i];
-        p.ow[t * p.n_k + i] = p.decay_kind == 1 ? expf(-expf(z)) : expf(logsigmoid_(z) * p.inv_tau);      // sigmoid(z)^(1/tau)
+        p.ow[t * p.n_k + i] = expf(logsigmoid_(p.z[t * p.z_stride + i]) * p.inv_tau);      // sigmoid(z)^(1/tau)
+    }
+    for (int64_t i = threadIdx.x; i < p.n_v; i += 256) p.ov[t * p.n_v + i] = ldf((const A*)p.v, t * p.v_stride + i);
+}
+
+// The operands of the RWKV time mix from its projections: r, k, v as they are and the decay of every key channel,
+//   w = exp(-exp(w0 + W2 tanh(l))),   l: the token's low-rank decay input [rank], W2 [n_k, rank],
+// with the rank-sized product inside (fp32 throughout; tanh(l) sits in LDS).
+struct WkvPrepArgs {
+    const void *r, *k, *v, *l;
+    int64_t r_stride, k_stride, v_stride, l_stride;
+    const void *w2, *w0;
+    float *oq, *ok, *ow, *ov;
+    int64_t n_k, n_v;
+    int rank;
+};
+
+template <typename A>
+__global__ __launch_bounds__(256) void wkv_prep_kernel(WkvPrepArgs p) {
+    extern __shared__ float th[];
+    const int64_t t = blockIdx.x;
+    for (int j = threadIdx.x; j < p.rank; j += 256) th[j] = tanhf(ldf((const A*)p.l, t * p.l_stride + j));
+    __syncthreads();
+    for (int64_t i = threadIdx.x; i < p.n_k; i += 256) {
+        const A* wr = (const A*)p.w2 + i * p.rank;
+        float z = ldf((const A*)p.w0, i);
+        for (int j = 0; j < p.rank; ++j) z = __builtin_fmaf((float)wr[j], th[j], z);
+        p.oq[t * p.n_k + i] = ldf((const A*)p.r, t * p.r_stride + i);
+        p.ok[t * p.n_k + i] = ldf((const A*)p.k, t * p.k_stride + i);
+        p.ow[t * p.n_k + i] = expf(-expf(z));
     }
     for (int64_t i = threadIdx.x; i < p.n_v; i += 256) p.ov[t * p.n_v + i] = ldf((const A*)p.v, t * p.v_stride + i);
 }
@@ -680,16 +707,30 @@ extern "C" int32_t nvh_hgrn2_prep(const void* q, int64_t q_stride, const void* f
 
 extern "C" int32_t nvh_gla_prep(const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v, int64_t v_stride,
                                 const float* decay_logits, int64_t z_stride, float q_scale, float tau, float* out_q, float* out_k,
-                                float* out_w, float* out_v, int64_t num_tokens, int64_t n_k, int64_t n_v, int32_t decay_kind, int32_t act_f32,
-                                nvh_stream_t stream) {
+                                float* out_w, float* out_v, int64_t num_tokens, int64_t n_k, int64_t n_v, int32_t act_f32, nvh_stream_t stream) {
     NVH_REQUIRE(q && k && v && decay_logits && out_q && out_k && out_w && out_v, NVH_EINVAL, "nvh_gla_prep: null pointer");
-    NVH_REQUIRE(num_tokens >= 0 && n_k > 0 && n_v > 0 && tau > 0.f && (decay_kind == 0 || decay_kind == 1), NVH_EINVAL, "nvh_gla_prep: bad sizes");
+    NVH_REQUIRE(num_tokens >= 0 && n_k > 0 && n_v > 0 && tau > 0.f, NVH_EINVAL, "nvh_gla_prep: bad sizes");
     if (num_tokens == 0) return NVH_OK;
-    const GlaPrepArgs p{q, k, v, q_stride, k_stride, v_stride, decay_logits, z_stride, q_scale, 1.0f / tau, out_q, out_k, out_w, out_v, n_k, n_v, decay_kind};
+    const GlaPrepArgs p{q, k, v, q_stride, k_stride, v_stride, decay_logits, z_stride, q_scale, 1.0f / tau, out_q, out_k, out_w, out_v, n_k, n_v};
     hipStream_t st = (hipStream_t)stream;
     if (act_f32) gla_prep_kernel<float><<<dim3((unsigned)num_tokens), 256, 0, st>>>(p);
     else gla_prep_kernel<bf16><<<dim3((unsigned)num_tokens), 256, 0, st>>>(p);
     NVH_CHECK_LAUNCH("nvh_gla_prep");
+    return NVH_OK;
+}
+
+extern "C" int32_t nvh_wkv_prep(const void* r, int64_t r_stride, const void* k, int64_t k_stride, const void* v, int64_t v_stride, const void* lowrank,
+                                int64_t lowrank_stride, const void* w2, const void* w0, float* out_q, float* out_k, float* out_w, float* out_v,
+                                int64_t num_tokens, int64_t n_k, int64_t n_v, int64_t rank, int32_t act_f32, nvh_stream_t stream) {
+    NVH_REQUIRE(r && k && v && lowrank && w2 && w0 && out_q && out_k && out_w && out_v, NVH_EINVAL, "nvh_wkv_prep: null pointer");
+    NVH_REQUIRE(num_tokens >= 0 && n_k > 0 && n_v > 0 && rank > 0 && rank <= 8192 && lowrank_stride >= rank, NVH_EINVAL, "nvh_wkv_prep: bad sizes");
+    if (num_tokens == 0) return NVH_OK;
+    const WkvPrepArgs p{r, k, v, lowrank, r_stride, k_stride, v_stride, lowrank_stride, w2, w0, out_q, out_k, out_w, out_v, n_k, n_v, (int)rank};
+    hipStream_t st = (hipStream_t)stream;
+    const size_t lds = sizeof(float) * (size_t)rank;
+    if (act_f32) wkv_prep_kernel<float><<<dim3((unsigned)num_tokens), 256, lds, st>>>(p);
+    else wkv_prep_kernel<bf16><<<dim3((unsigned)num_tokens), 256, lds, st>>>(p);
+    NVH_CHECK_LAUNCH("nvh_wkv_prep");
     return NVH_OK;
 }
 

@@ -287,7 +287,7 @@ __global__ __launch_bounds__(256) void residual_postnorm_kernel(PostNormArgs p) 
 }
 
 // y = act(g) (* u when gated): g = columns [0, inter) and u = columns [inter, 2 inter) of the row.
-// act: 0 silu, 1 gelu (tanh form), 2 squared relu, 3 tanh.
+// act: 0 silu, 1 gelu (tanh form), 2 squared relu.
 template <typename A>
 __global__ __launch_bounds__(256) void act_mul_kernel(const A* __restrict__ gu, int64_t gu_stride, A* __restrict__ y, int64_t y_stride, int64_t rows, int inter,
                                                       int act, int gated) {
@@ -299,8 +299,7 @@ __global__ __launch_bounds__(256) void act_mul_kernel(const A* __restrict__ gu, 
     float v;
     if (act == 0) v = g / (1.0f + expf(-g));
     else if (act == 1) v = 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
-    else if (act == 2) v = g > 0.f ? g * g : 0.f;
-    else v = tanhf(g);
+    else v = g > 0.f ? g * g : 0.f;
     if (gated) v *= ldf(gu, row * gu_stride + inter + c);
     y[row * y_stride + c] = (A)v;
 }
@@ -489,7 +488,7 @@ extern "C" int32_t nvh_residual_postnorm(const void* y, int64_t y_stride, const 
 
 extern "C" int32_t nvh_act_mul(const void* x, int64_t row_stride, void* y, int64_t y_stride, int64_t rows, int64_t inter, int32_t act, int32_t gated,
                                int32_t act_f32, nvh_stream_t stream) {
-    NVH_STREAM_ARGS_OK("nvh_act_mul", x && y && rows >= 0 && inter > 0 && act >= 0 && act <= 3 && row_stride >= (gated ? 2 : 1) * inter && y_stride >= inter);
+    NVH_STREAM_ARGS_OK("nvh_act_mul", x && y && rows >= 0 && inter > 0 && act >= 0 && act <= 2 && row_stride >= (gated ? 2 : 1) * inter && y_stride >= inter);
     if (rows == 0) return NVH_OK;
     hipStream_t st = (hipStream_t)stream;
     const unsigned blocks = (unsigned)nvh_cdiv(rows * inter, 256);

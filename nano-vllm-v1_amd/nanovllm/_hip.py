@@ -113,7 +113,8 @@ SIGNATURES = {
     "nvh_gated_linear_scan": (i32, [vp, i64, vp, i64, i64, vp, i64, i32, vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, vp, i32, vp, vp]),
     "nvh_scan_segmentable": (i32, [i64]),
     "nvh_hgrn2_prep": (i32, [vp, i64, vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, i64, i64, i64, i32, vp]),
-    "nvh_gla_prep": (i32, [vp, i64, vp, i64, vp, i64, vp, i64, f32, f32, vp, vp, vp, vp, i64, i64, i64, i32, i32, vp]),
+    "nvh_gla_prep": (i32, [vp, i64, vp, i64, vp, i64, vp, i64, f32, f32, vp, vp, vp, vp, i64, i64, i64, i32, vp]),
+    "nvh_wkv_prep": (i32, [vp, i64, vp, i64, vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp]),
     "nvh_token_shift_mix": (i32, [vp, i64, vp, vp, vp, vp, i64, vp, vp, i64, i64, i64, i32, vp]),
     "nvh_rotary_qkv_prep": (i32, [vp, i64, vp, i64, vp, i64, vp, vp, f32, i64, i32, f32, f32, vp, vp, vp, i64, i64, i64, i64, i32, vp]),
     "nvh_ssd_conv_prep": (i32, [vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, vp, vp, vp, vp, i32, vp]),

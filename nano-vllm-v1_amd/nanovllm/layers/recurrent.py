@@ -234,13 +234,13 @@ class WKV(nn.Module):
         super().__init__()
         n = num_heads * head_dim
         self.num_heads, self.head_dim, self.rank, self.eps = num_heads, head_dim, rank, eps
-        self.decay_up = MergedLinear(rank, [n], bias=True)                 # W2 and w0
+        self.w2 = nn.Parameter(torch.zeros(n, rank), requires_grad=False)
+        self.w0 = nn.Parameter(torch.zeros(n), requires_grad=False)
         self.bonus = nn.Parameter(torch.zeros(num_heads, head_dim, dtype=torch.float32), requires_grad=False)      # (an operand of the fp32 scan)
         self.norm = nn.Parameter(torch.ones(n), requires_grad=False)
         self.memory = DiagonalDecayRecurrence(num_heads, head_dim, head_dim, state_runs=state_runs)
 
     def forward(self, r, k, v, gate, lowrank, run: int = 0) -> torch.Tensor:
-        z = self.decay_up(ops.act_mul(lowrank, "tanh", False), out_f32=True)
-        oq, ok, ow, ov = ops.gla_prep(r, k, v, z, 1.0, decay="exp_exp")
+        oq, ok, ow, ov = ops.wkv_prep(r, k, v, lowrank, self.w2.data, self.w0.data)
         o = self.memory(oq, ok, ow, ov, run, read_first=True, bonus=self.bonus.data)
         return ops.group_rmsnorm_gate(o, self.norm.data, self.head_dim, self.eps, gate, "silu", gate_first=False)

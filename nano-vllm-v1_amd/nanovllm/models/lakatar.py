@@ -192,7 +192,7 @@ class LakatarForCausalLM(nn.Module):
                 return pm + "shift.mu", leaf[3:]
             if leaf in ("r", "k", "v", "g", "w1"):
                 return pm + leaf + ".weight", None
-            direct = {"w2": "cell.decay_up.weight", "w0": "cell.decay_up.bias", "u": "cell.bonus", "norm": "cell.norm"}
+            direct = {"w2": "cell.w2", "w0": "cell.w0", "u": "cell.bonus", "norm": "cell.norm"}
             if leaf in direct:
                 return pm + direct[leaf], None
         elif isinstance(mixer, LakatarLatentAttention):

@@ -736,7 +736,7 @@ def delta_post(o: torch.Tensor, norm_weight: torch.Tensor, gate: torch.Tensor | 
 
 # ---------------------------------------------------------------- layer norm / RMS norm around the fp32 stream, plain activations
 NORM_KINDS = {None: 0, "layer": 1, "rms": 2}
-ACTS = {"silu": 0, "gelu_tanh": 1, "relu2": 2, "tanh": 3}
+ACTS = {"silu": 0, "gelu_tanh": 1, "relu2": 2}
 
 
 def embedding_pos_stream(ids: torch.Tensor, positions: torch.Tensor, table: torch.Tensor, pos_table: torch.Tensor | None, scale: float = 1.0) -> torch.Tensor:
@@ -791,7 +791,7 @@ def residual_postnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, y=None,
 
 
 def act_mul(x: torch.Tensor, act: str, gated: bool) -> torch.Tensor:
-    """act(x) for plain rows, act(x[:, :I]) * x[:, I:] for a merged [gate | up] projection; act: silu, gelu_tanh, relu2, tanh."""
+    """act(x) for plain rows, act(x[:, :I]) * x[:, I:] for a merged [gate | up] projection; act: silu, gelu_tanh, relu2."""
     f = _act_flag(x)
     assert x.dim() == 2 and x.stride(1) == 1
     rows, inter = x.shape[0], x.shape[1] // 2 if gated else x.shape[1]
@@ -866,9 +866,8 @@ def hgrn2_prep(q, f, v, f_bias, lower):
     return oq, ok, ow, ov
 
 
-def gla_prep(q, k, v, decay_logits, q_scale: float, tau: float = 1.0, decay: str = "sigmoid_pow"):
-    """fp32 (q * q_scale, k, w, v) from projection columns and fp32 decay logits z: w = sigmoid(z)^(1/tau) ("sigmoid_pow") or
-    exp(-exp(z)) ("exp_exp")."""
+def gla_prep(q, k, v, decay_logits, q_scale: float, tau: float):
+    """fp32 (q * q_scale, k, sigmoid(decay_logits)^(1/tau), v) from projection columns and fp32 decay logits."""
     fl = _act_flag(q, k, v)
     t, nk, nv = q.shape[0], q.shape[1], v.shape[1]
     assert q.stride(1) == 1 and k.stride(1) == 1 and v.stride(1) == 1 and k.shape == (t, nk)
@@ -876,8 +875,22 @@ def gla_prep(q, k, v, decay_logits, q_scale: float, tau: float = 1.0, decay: str
     oq, ok, ow = (torch.empty(t, nk, dtype=F32, device=q.device) for _ in range(3))
     ov = torch.empty(t, nv, dtype=F32, device=q.device)
     _hip.call("nvh_gla_prep", q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), decay_logits.data_ptr(),
-              decay_logits.stride(0), float(q_scale), float(tau), oq.data_ptr(), ok.data_ptr(), ow.data_ptr(), ov.data_ptr(), t, nk, nv,
-              {"sigmoid_pow": 0, "exp_exp": 1}[decay], fl, _stream())
+              decay_logits.stride(0), float(q_scale), float(tau), oq.data_ptr(), ok.data_ptr(), ow.data_ptr(), ov.data_ptr(), t, nk, nv, fl, _stream())
+    return oq, ok, ow, ov
+
+
+def wkv_prep(r, k, v, lowrank, w2, w0):
+    """fp32 (r, k, w, v) of the RWKV time mix from projection columns: w = exp(-exp(w0 + w2 @ tanh(lowrank))) per key channel, the
+    rank-sized product formed in fp32 inside the launch."""
+    fl = _act_flag(r, k, v, lowrank, w2, w0)
+    t, nk, nv = r.shape[0], r.shape[1], v.shape[1]
+    rank = lowrank.shape[1]
+    assert r.stride(1) == 1 and k.stride(1) == 1 and v.stride(1) == 1 and lowrank.stride(1) == 1 and k.shape == (t, nk) and lowrank.shape[0] == t
+    assert w2.is_contiguous() and tuple(w2.shape) == (nk, rank) and w0.is_contiguous() and w0.numel() == nk
+    oq, ok, ow = (torch.empty(t, nk, dtype=F32, device=r.device) for _ in range(3))
+    ov = torch.empty(t, nv, dtype=F32, device=r.device)
+    _hip.call("nvh_wkv_prep", r.data_ptr(), r.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), lowrank.data_ptr(), lowrank.stride(0),
+              w2.data_ptr(), w0.data_ptr(), oq.data_ptr(), ok.data_ptr(), ow.data_ptr(), ov.data_ptr(), t, nk, nv, rank, fl, _stream())
     return oq, ok, ow, ov
 
 
