@@ -508,15 +508,14 @@ def _lakatar_cfg(z):
     mixers = [("wkv", {"heads": w // 64, "dim": 64}), ("latent_attention", latent), ("retention", retention)]
     moe = {"kind": "moe", "expert": {"ff": z["ff"] // 8}, "router": {"experts": 16, "top": 2, "scale": 1.0, "groups": {"count": 4, "keep": 2}},
            "shared": {"ff": z["ff"] // 4}}
-    layers, first_latent = [], None
+    layers, latent_layers = [], []
     for i in range(z["layers"]):
         kind, mixer = mixers[i % 3]
         mixer = dict(mixer)
         if kind == "latent_attention":
-            if first_latent is None:
-                first_latent = i
-            elif "kv_from" not in layers[first_latent]["mixer"] and sum(l["type"] == kind for l in layers) == 1:
-                mixer["kv_from"] = first_latent
+            if len(latent_layers) == 1:                      # the second one reads the first one's latent
+                mixer["kv_from"] = latent_layers[0]
+            latent_layers.append(i)
         layers.append({"type": kind, "mixer": mixer, "mlp": moe})
     return {"architecture": "Lakatar", "vocab": z["vocab"], "width": w, "norm": {"eps": 1e-6}, "postln_alpha": 2.0, "layers": layers}
 

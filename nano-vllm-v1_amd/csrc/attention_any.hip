@@ -12,6 +12,9 @@
 //                         Optional: a distance bias, score -= slope[head] * (query position - key position), and a
 //                         sliding window that keeps the first tokens: query i sees key j <= i when i - j < window or
 //                         j < keep_first; key tiles that no query of a workgroup can see are never loaded.
+//                         Steps in which every sequence brings one query: the heads that share a KV head share a workgroup
+//                         (groups of more than 16 heads in parts); when that leaves most of the chip idle, a sequence's key
+//                         tiles are dealt out to several workgroups whose rows a second launch merges.
 // Activations and caches are of type A (bf16 or fp32).  Key tiles always start at key 0 of a sequence and every query
 // row keeps its own running maximum and sum, so a query's result does not depend on how the prompt was cut into steps
 // or on what else is in the batch.

@@ -19,6 +19,7 @@ from torch import nn
 
 from .. import ops
 from ..utils.context import get_context
+from .linear import MergedLinear
 
 
 def store_kvcache(key: torch.Tensor, value: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
@@ -172,7 +173,6 @@ class LatentAttention(nn.Module):
                  freq: torch.Tensor | None, mag: float = 1.0, interleaved: bool = True, gated: bool = True, cache_runs: int = 1,
                  kv_source: "LatentAttention | None" = None):
         super().__init__()
-        from .linear import MergedLinear
         self.num_heads, self.qk_dim, self.rot_dim, self.v_dim, self.q_rank, self.kv_rank = num_heads, head_dim, rot_dim, value_dim, q_rank, kv_rank
         self.scale, self.eps, self.mag, self.interleaved, self.gated = scale, eps, mag, interleaved, gated
         self.q_norm = nn.Parameter(torch.ones(q_rank), requires_grad=False)
