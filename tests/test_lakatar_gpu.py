@@ -307,7 +307,7 @@ def test_router_by_scores_with_correction_groups_and_scale():
     from nanovllm import ops
     g = torch.Generator().manual_seed(1)
     for E, top, groups, keep, scale in [(6, 2, 3, 2, 2.5), (7, 3, 1, 1, 1.0), (8, 4, 4, 2, 0.7), (64, 6, 8, 3, 1.0), (130, 8, 10, 4, 1.5), (3, 3, 3, 3, 1.0),
-                                        (12, 2, 4, 1, 1.0), (1, 1, 1, 1, 2.0)]:
+                                        (12, 2, 4, 1, 1.0), (1, 1, 1, 1, 2.0), (300, 5, 10, 3, 1.0)]:
         x, w = torch.randn(33, 70, generator=g), torch.randn(E, 70, generator=g) * 0.3
         corr = torch.randn(E, generator=g) * 0.2 - 0.3          # mostly negative: zeros in place of minus infinity would win
         aux = torch.randn(2, 70, generator=g)
