@@ -516,7 +516,8 @@ int32_t nvh_gemm_any_nt(const void* x, int64_t x_row_stride, const void* w, cons
 
 /* Attention with a norm over the whole projection, partial rotary, rotated values and a per-head output gate.
  * nvh_attn_rotary_prep reads the fused projection row [q (H dim) | k (G dim) | v (G vdim) | gate (H, when gate_out)] of
- * every token: RMS norm (eps, weights of the full projection size; both NULL: no norm) over all of q and all of k; the first rot_dims
+ * every token: RMS norm (eps, weights of the full projection size; both NULL: no norm) over all of q and all of k - or, with
+ * norm_per_head, over every head by itself with weights of size dim that the heads share; the first rot_dims
  * dimensions of every q / k head are turned by position * qk_freq[pair] with cos and sin scaled by qk_mag (pairs are
  * (i, i + rot_dims/2), or (2i, 2i+1) when interleaved; the frequency table carries any scaling rule); the value is
  * turned by its position over all vdim dimensions with v_freq (NULL: stored as it is).  q -> q_out [T, H dim], k and v ->
@@ -526,7 +527,7 @@ int32_t nvh_attn_rotary_prep(const void* proj, int64_t proj_row_stride, const vo
                              float eps, const int64_t* positions, const float* qk_freq, float qk_mag, int64_t rot_dims,
                              int32_t qk_interleaved, const float* v_freq, int32_t v_interleaved, void* q_out, float* gate_out,
                              void* k_cache, void* v_cache, const int32_t* slot_mapping, int64_t page, int64_t num_tokens,
-                             int64_t num_q_heads, int64_t num_kv_heads, int64_t dim, int64_t vdim, int32_t act_f32,
+                             int64_t num_q_heads, int64_t num_kv_heads, int64_t dim, int64_t vdim, int32_t norm_per_head, int32_t act_f32,
                              nvh_stream_t stream);
 /* Causal softmax attention of var-len queries (cu_seqlens_q NULL: one per sequence) over the paged caches
  * [pages, page, G, dim] / [pages, G, vdim, page]; context_lens counts the keys including this step's.  Scores, weights
@@ -534,30 +535,43 @@ int32_t nvh_attn_rotary_prep(const void* proj, int64_t proj_row_stride, const vo
  * multiplied by gate[t, h] (NULL: none).  out [T, H vdim] of type A.
  * slopes (fp32 [H], NULL: none): a distance bias, score -= slopes[h] * (query position - key position).
  * window > 0: query i sees key j <= i only when i - j < window or j < keep_first (the first tokens stay visible and
- * their distance is counted from where they stand); key tiles no query of a workgroup can see are skipped.  window 0: plain causal attention. */
+ * their distance is counted from where they stand); key tiles no query of a workgroup can see are skipped.  window 0: plain causal attention.
+ * chunk > 0: query i sees key j <= i only when j >= (i / chunk) chunk (blocks of `chunk` positions counted from the sequence's start).
+ * sinks (fp32 [H], NULL: none): exp(sinks[h]) joins the softmax's denominator of every row of head h once (no key, no value, not scaled). */
 int32_t nvh_attn_paged_any(const void* q, const void* k_cache, const void* v_cache, const int32_t* cu_seqlens_q,
                            const int32_t* context_lens, const int32_t* block_tables, int64_t table_stride, int64_t batch,
                            int64_t total_q, int64_t page, int64_t num_q_heads, int64_t num_kv_heads, int64_t dim, int64_t vdim,
                            float scale, const float* gate, const float* v_freq, int32_t v_interleaved, const float* slopes,
-                           int64_t window, int64_t keep_first, void* out, float* parts_ws, int64_t parts_ws_bytes, int32_t act_f32, nvh_stream_t stream);
+                           int64_t window, int64_t keep_first, int64_t chunk, const float* sinks, void* out, float* parts_ws, int64_t parts_ws_bytes,
+                           int32_t act_f32, nvh_stream_t stream);
 /* Bytes of fp32 scratch (parts_ws) with which nvh_attn_paged_any spreads the key tiles of one-query steps over several workgroups
  * when the launch would otherwise leave most of the chip idle (0: none wanted; without scratch the launch is the plain one). */
 int64_t nvh_attn_paged_any_parts_bytes(int64_t batch, int64_t total_q, int64_t num_q_heads, int64_t num_kv_heads, int64_t dim, int64_t vdim,
                                        int64_t page, int32_t turned_back, int32_t act_f32);
 
 /* Generalized delta rule, state [slots, H, dk, dv] fp32:  S <- diag(w) S - (a u)(u^T S) + k v^T,  o = S^T r.
- * nvh_delta_prep: out fp32 [T, H, 6, dk] = r | k | w | u | a u | v per head, with w = exp(-decay_scale sigmoid(w0 + w2 tanh(lowrank))),
+ * nvh_delta_prep: out fp32 [T, H, 5 dk + dv] = r | k | w | u | a u (dk each) | v (dv) per head, here with dv = dk, with w = exp(-decay_scale sigmoid(w0 + w2 tanh(lowrank))),
  * a = sigmoid(a_raw + a_bias), u = k / sqrt(sum_head k^2 + 1e-6) (value size = key size dk).
  * nvh_delta_scan: sequence b owns state slot slots[b] (< 0: a padded row) and this step's tokens cu_seqlens_q[b] ..
  * (NULL: row b); it starts from zero when context_lens[b] equals its token count, else from the slot, and leaves the
- * state there; out fp32 [T, H dk].  dk <= 256.
- * nvh_delta_post: y (type A) = o / rms_head(o) * norm_weight * sigmoid(gate) (gate NULL: none). */
+ * state there; out fp32 [T, H dv].  dk <= 256.
+ * nvh_delta_post: y (type A) = o / rms_head(o) * norm_weight * sigmoid(gate) (gate NULL: none).
+ * nvh_gated_delta_prep: the scan's rows for the gated delta rule, S <- g S; d = beta (v - S^T k); S <- S + k d^T; o = S^T q (the
+ * recurrence above with w = g on every channel, u = k, a u = beta g k and the written key beta k).  qkv: the channels q | k
+ * (qk_heads dk each; value head h reads q / k head h / (heads / qk_heads)) | v (heads dv) of the projection row; they pass a causal
+ * convolution (conv_w [C, taps], last tap on the current token, continued from conv_state [slots, taps - 1, C], zeros at a
+ * sequence's start; nvh_conv_state_update afterwards) and silu; q and k become unit vectors per head (x / sqrt(sum x^2 + 1e-6)),
+ * q also times dk^-1/2; beta = sigmoid(b), g = exp(-exp(a_log) softplus(a + dt_bias)) per head.  All arithmetic in fp32. */
+int32_t nvh_gated_delta_prep(const void* qkv, int64_t qkv_stride, const void* b, int64_t b_stride, const void* a, int64_t a_stride,
+                             const void* conv_w, const void* dt_bias, const void* a_log, const float* conv_state, const int32_t* slots,
+                             const int32_t* cu_seqlens_q, const int32_t* context_lens, float* out, int64_t batch, int64_t num_tokens,
+                             int64_t taps, int64_t heads, int64_t qk_heads, int64_t dk, int64_t dv, int32_t act_f32, nvh_stream_t stream);
 int32_t nvh_delta_prep(const void* r, int64_t r_stride, const void* k, int64_t k_stride, const void* v, int64_t v_stride,
                        const void* a_raw, int64_t a_stride, const void* lowrank, int64_t lowrank_stride,
                        const void* w2, const void* w0, const void* a_bias, float* out, int64_t num_tokens, int64_t heads, int64_t dk,
                        int64_t rank, float decay_scale, int32_t act_f32, nvh_stream_t stream);
 int32_t nvh_delta_scan(const float* pack, float* state, const int32_t* slots, const int32_t* cu_seqlens_q,
-                       const int32_t* context_lens, float* out, int64_t batch, int64_t heads, int64_t dk, nvh_stream_t stream);
+                       const int32_t* context_lens, float* out, int64_t batch, int64_t heads, int64_t dk, int64_t dv, nvh_stream_t stream);
 int32_t nvh_delta_post(const float* o, const void* norm_weight, const void* gate, int64_t gate_stride, void* y, int64_t y_stride,
                        int64_t rows, int64_t heads, int64_t dv, float eps, int32_t act_f32, nvh_stream_t stream);
 
@@ -582,6 +596,12 @@ int32_t nvh_residual_norm(const void* a, int64_t a_stride, const void* a_weight,
 int32_t nvh_residual_postnorm(const void* y, int64_t y_stride, const float* y32, int64_t y32_stride, const void* layer_scale, float alpha,
                               float* x, int32_t write_x, const void* norm_weight, float weight_offset, float eps, void* h, int64_t h_stride,
                               int64_t rows, int64_t dim, int32_t act_f32, nvh_stream_t stream);
+/* The close of a sublayer whose result is normed before it joins the stream.  Per row:
+ *   y = a_scale a + b_scale b + c32;   x <- x + mult * weight * y / sqrt(mean(y^2) + eps);   h <- x (type A; NULL: not wanted)
+ * a, b (type A) and c32 (fp32) may be NULL (not all); weight (type A): one number (weight_elems 1) or [dim].  fp32 arithmetic. */
+int32_t nvh_residual_subnorm(const void* a, int64_t a_stride, float a_scale, const void* b, int64_t b_stride, float b_scale, const float* c32,
+                             int64_t c32_stride, float mult, const void* weight, int64_t weight_elems, float eps, float* x, void* h,
+                             int64_t h_stride, int64_t rows, int64_t dim, int32_t act_f32, nvh_stream_t stream);
 /* y[rows, inter] = act(x[:, :inter]) (* x[:, inter:2 inter] when gated), evaluated in fp32.  act 0: silu, 1: gelu (tanh form),
  * 2: squared relu. */
 int32_t nvh_act_mul(const void* x, int64_t row_stride, void* y, int64_t y_stride, int64_t rows, int64_t inter, int32_t act, int32_t gated,
@@ -613,6 +633,9 @@ int32_t nvh_logits_scale(const void* logits, int64_t row_stride, float* out, int
  * [slots, taps - 1, C] (zeros at a sequence's start), then silu -> out_x [T, inner], out_b, out_c [T, gn];
  * out_dt = softplus(dt + dt_bias) and out_decay = exp(-exp(a_log) out_dt), both [T, H].
  * nvh_conv_state_update (after nvh_ssd_conv_prep of the same step): the last taps - 1 inputs of every sequence -> its slot.
+ * nvh_stream_conv: h_t (type A) = x_t + sum_k w[:, k] x_(t - taps + 1 + k) over the fp32 stream x [T, dim] (w [dim, taps], type A, last tap
+ * on the token itself), continued from state fp32 [slots, taps - 1, dim] (zeros at a sequence's start); nvh_conv_state_update
+ * over x (as fp32 input) afterwards leaves every sequence's last taps - 1 rows in its slot.
  * nvh_group_rmsnorm_gate: y (type A) = unit over groups of group_size columns of o (o * gate first when gate_first),
  * times weight ([group_size] shared, or [groups group_size] when weight_full; NULL: none), times gate afterwards otherwise;
  * gate_act 0: no gate, 1: sigmoid(gate), 2: silu(gate). */
@@ -649,6 +672,9 @@ int32_t nvh_ssd_conv_prep(const void* xbc, int64_t xbc_stride, const void* dt, i
                           nvh_stream_t stream);
 int32_t nvh_conv_state_update(const void* xbc, int64_t xbc_stride, float* conv_state, const int32_t* slots, const int32_t* cu_seqlens_q,
                               const int32_t* context_lens, int64_t batch, int64_t taps, int64_t channels, int32_t act_f32, nvh_stream_t stream);
+int32_t nvh_stream_conv(const float* x, const void* w, const float* state, const int32_t* slots, const int32_t* cu_seqlens_q,
+                        const int32_t* context_lens, void* h, int64_t h_stride, int64_t batch, int64_t num_tokens, int64_t taps, int64_t dim,
+                        int32_t act_f32, nvh_stream_t stream);
 int32_t nvh_group_rmsnorm_gate(const float* o, const void* weight, int32_t weight_full, const void* gate, int64_t gate_stride,
                                int32_t gate_act, int32_t gate_first, void* y, int64_t y_stride, int64_t rows, int64_t groups,
                                int64_t group_size, float eps, int32_t act_f32, nvh_stream_t stream);
@@ -659,14 +685,20 @@ int32_t nvh_group_rmsnorm_gate(const float* o, const void* weight, int32_t weigh
  * (tile_expert, tile_row0, tile_rows; unused tiles have 0 rows); max_tiles >= nvh_moe_max_tiles(T top, E).
  * nvh_gemm_grouped_any_nt: y[pos] = x[gather ? gather[pos] : pos] w[expert]^T over the tiles, w [E, N, K]; types as
  * nvh_gemm_any_nt.  nvh_moe_combine: out fp32 [T, dim] = sum_r weights[t, r] y[pos_of_pair[t, r]] (+ shared[t], type A,
- * times sigmoid(shared_gate[t shared_gate_stride]) when a gate logit per token is given). */
+ * times sigmoid(shared_gate[t shared_gate_stride]) when a gate logit per token is given; weights NULL: all 1). */
 int32_t nvh_moe_route(const float* logits, int64_t row_stride, int32_t* ids, float* weights, int64_t num_tokens, int64_t experts,
                       int64_t top, nvh_stream_t stream);
 /* nvh_moe_route with the router's product inside: logits = x w^T + bias (x [T, K], w [E, K], bias [E] or NULL, type A;
- * products and sums in fp32), optionally written to logits_out fp32 [T, E]. */
+ * products and sums in fp32), optionally written to logits_out fp32 [T, E].  sigmoid_scores: the weights are the picked
+ * experts' own sigmoid(logit), not renormalised (the choice by logit is the choice by score). */
 int32_t nvh_moe_route_linear(const void* x, int64_t x_row_stride, const void* w, const void* bias, int32_t* ids, float* weights,
-                             float* logits_out, int64_t num_tokens, int64_t experts, int64_t K, int64_t top, int32_t act_f32,
-                             nvh_stream_t stream);
+                             float* logits_out, int64_t num_tokens, int64_t experts, int64_t K, int64_t top, int32_t sigmoid_scores,
+                             int32_t act_f32, nvh_stream_t stream);
+/* The experts' activation where the routing weight multiplies the expert's input: over the rows gate_up[pos] = [G | U] of the first
+ * grouped product (formed from the unweighted tokens), for every pair with pos = pos_of_pair[pair] >= 0 and w = weights[pair]
+ * (NULL: 1):  g = min(w G, limit), u = clamp(w U, -limit, limit), y[pos] = g sigmoid(alpha g) (u + 1).  fp32 arithmetic. */
+int32_t nvh_glu_clamp_pairs(const void* gate_up, int64_t row_stride, const int32_t* pos_of_pair, const float* weights, void* y, int64_t y_stride,
+                            int64_t pairs, int64_t inter, float limit, float alpha, int32_t act_f32, nvh_stream_t stream);
 int64_t nvh_moe_max_tiles(int64_t pairs, int64_t experts);
 int32_t nvh_moe_align(const int32_t* ids, int64_t num_tokens, int64_t experts, int64_t top, int32_t* src_token, int32_t* pos_of_pair,
                       int32_t* tile_expert, int32_t* tile_row0, int32_t* tile_rows, int64_t max_tiles, nvh_stream_t stream);

@@ -1,7 +1,8 @@
 // Paged causal attention for any head sizes (query/key size `dim`, value size `vdim`, any page size), with the pieces a
 // gated, value-rotating attention needs around it:
 //   nvh_attn_rotary_prep  per token, over the fused projection row [q | k | v | gate]: RMS norm over the WHOLE q and the
-//                         whole k projection (not per head), partial rotary on q and k (frequency table given by the
+//                         whole k projection, or over every head by itself with one weight row shared by the heads
+//                         (norm_per_head), partial rotary on q and k (frequency table given by the
 //                         caller, so any scaling rule fits), rotation of the value by its own position over all of
 //                         vdim, sigmoid of the per-head gate; q goes to a packed buffer, k and v to their cache slots.
 //                         Keys are cached [pages, page, G, dim]; values TRANSPOSED within a page, [pages, G, vdim, page],
@@ -12,6 +13,10 @@
 //                         Optional: a distance bias, score -= slope[head] * (query position - key position), and a
 //                         sliding window that keeps the first tokens: query i sees key j <= i when i - j < window or
 //                         j < keep_first; key tiles that no query of a workgroup can see are never loaded.
+//                         Optional: chunks, query i sees key j <= i only when both lie in the same block of `chunk`
+//                         positions counted from the sequence's start; and a sink per head, a learned logit that joins the
+//                         softmax's denominator once, unscaled, with no key and no value (it is the state a row starts from:
+//                         maximum = sink, sum = 1, output = 0).
 //                         Steps in which every sequence brings one query: the heads that share a KV head share a workgroup
 //                         (groups of more than 16 heads in parts); when that leaves most of the chip idle, a sequence's key
 //                         tiles are dealt out to several workgroups whose rows a second launch merges.
@@ -38,7 +43,8 @@ __device__ __forceinline__ float block_sum_256(float v, float* scratch) {
 struct PrepArgs {
     const void* proj;          // [T, ld] : q (H*dim) | k (G*dim) | v (G*vdim) | gate (H)
     int64_t ld;
-    const void *q_norm, *k_norm;   // [H*dim], [G*dim]
+    const void *q_norm, *k_norm;   // [H*dim], [G*dim]; norm_per_head: [dim] each, shared by the heads
+    int norm_per_head;
     float eps;
     const int64_t* positions;
     const float* qk_freq;      // [rot_dims / 2]
@@ -56,6 +62,7 @@ struct PrepArgs {
 template <typename A>
 __global__ __launch_bounds__(256) void attn_rotary_prep_kernel(PrepArgs a) {
     __shared__ float red[4];
+    extern __shared__ float head_inv[];                      // norm_per_head: 1 / rms of every q head, then of every k head
     const int64_t t = blockIdx.x;
     const A* row = (const A*)a.proj + t * a.ld;
     const int nq = a.H * a.dim, nk = a.G * a.dim, nv = a.G * a.vdim;
@@ -63,7 +70,20 @@ __global__ __launch_bounds__(256) void attn_rotary_prep_kernel(PrepArgs a) {
     const A* kr = row + nq;
     const A* vr = kr + nk;
     float inv_q = 1.f, inv_k = 1.f;
-    if (a.q_norm) {                                          // (null norm weights: q and k pass as they are)
+    if (a.q_norm && a.norm_per_head) {                       // a wave per head in turn (q heads, then k heads: they lie one after the other)
+        const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+        for (int h = wave; h < a.H + a.G; h += 4) {
+            const A* hr = qr + (int64_t)h * a.dim;
+            float ss = 0.f;
+            for (int i = lane; i < a.dim; i += 64) {
+                const float v = ldf(hr, i);
+                ss += v * v;
+            }
+            ss = wave_sum(ss);
+            if (lane == 0) head_inv[h] = 1.0f / sqrtf(ss / (float)a.dim + a.eps);
+        }
+        __syncthreads();
+    } else if (a.q_norm) {                                   // (null norm weights: q and k pass as they are)
         float sq = 0.f, sk = 0.f;
         for (int i = threadIdx.x; i < nq; i += 256) {
             const float v = ldf(qr, i);
@@ -85,17 +105,19 @@ __global__ __launch_bounds__(256) void attn_rotary_prep_kernel(PrepArgs a) {
         const A* src = which ? kr : qr;
         const A* wn = (const A*)(which ? a.k_norm : a.q_norm);
         const float inv = which ? inv_k : inv_q;
+        const int hbase = which ? a.H : 0;
         A* dst = which ? (slot >= 0 && a.k_cache ? (A*)a.k_cache + slot * nk : nullptr) : (A*)a.q_out + t * nq;
         if (!dst) continue;
         for (int i = threadIdx.x; i < n; i += 256) {
             const int d = i % a.dim;
-            float v = wn ? ldf(src, i) * inv * ldf(wn, i) : ldf(src, i);
+            const float rinv = a.norm_per_head && wn ? head_inv[hbase + i / a.dim] : inv;
+            float v = wn ? ldf(src, i) * rinv * ldf(wn, a.norm_per_head ? d : i) : ldf(src, i);
             if (d < a.rot_dims) {
                 int partner, pair;
                 bool first;
                 pair_of(d, a.rot_dims, a.qk_interleaved, partner, pair, first);
                 const int j = i - d + partner;
-                const float o = wn ? ldf(src, j) * inv * ldf(wn, j) : ldf(src, j);
+                const float o = wn ? ldf(src, j) * rinv * ldf(wn, a.norm_per_head ? partner : j) : ldf(src, j);
                 float sn, cs;
                 rot_sincos<A>(pos * a.qk_freq[pair], sn, cs);
                 const float c = cs * a.qk_mag, s = sn * a.qk_mag;
@@ -146,6 +168,8 @@ struct AttnArgs {
     void* out;                 // [T, H*vdim]
     const float* slopes;       // [H] or null: score -= slopes[head] * (query position - key position)
     int window, keep_first;    // window > 0: key j is visible to query i only when i - j < window or j < keep_first
+    int chunk;                 // chunk > 0: ... and only when j >= (i / chunk) * chunk
+    const float* sinks;        // [H] or null: a logit per head that joins the denominator of every row of that head
     int pages_offset;          // byte offset in LDS of the sequence's page ids (matrix-core kernel)
     int ml_offset;             // ... and of the waves' (max, sum) pairs in the one-query form
     int kv_split;              // one-query form: workgroups per (sequence, KV head), each with H / (G kv_split) of the group's heads
@@ -158,9 +182,11 @@ struct AttnArgs {
 // the first query on.  next(k0) is the start of the tile after k0.
 struct TileWalk {
     int first_end, win_start, tile;
-    __device__ __forceinline__ TileWalk(int window, int keep_first, int qlo, int tile_) : tile(tile_) {
+    __device__ __forceinline__ TileWalk(int window, int keep_first, int chunk, int qlo, int tile_) : tile(tile_) {
         first_end = window > 0 ? ((keep_first + tile_ - 1) / tile_) * tile_ : 0;
         win_start = window > 0 ? (max(qlo - window + 1, 0) / tile_) * tile_ : 0;
+        // (the chunk of the first query starts no later than any other query's: earlier tiles are seen by none)
+        if (chunk > 0) win_start = max(win_start, ((qlo / chunk) * chunk / tile_) * tile_);
     }
     __device__ __forceinline__ int next(int k0) const {
         const int n = k0 + tile;
@@ -168,8 +194,8 @@ struct TileWalk {
     }
 };
 
-__device__ __forceinline__ bool key_visible(int key, int qpos, int window, int keep_first) {
-    return key <= qpos && (window <= 0 || qpos - key < window || key < keep_first);
+__device__ __forceinline__ bool key_visible(int key, int qpos, int window, int keep_first, int chunk) {
+    return key <= qpos && (window <= 0 || qpos - key < window || key < keep_first) && (chunk <= 0 || key >= (qpos / chunk) * chunk);
 }
 
 template <typename A, int AVC>
@@ -211,12 +237,13 @@ __global__ __launch_bounds__(256) void attn_paged_any_kernel(AttnArgs a) {
     float acc[AVC];
 #pragma unroll
     for (int c = 0; c < AVC; ++c) acc[c] = 0.f;
-    float m_run = -INFINITY, l_run = 0.f;
+    // (a sink is what the row starts from: it has been seen with score sink, weight 1 and no value)
+    float m_run = a.sinks ? a.sinks[head] : -INFINITY, l_run = a.sinks ? 1.f : 0.f;
     const int qpos = past + q0 + qi;                         // this lane's query position (valid for qi < nq)
     const int last_key = past + q0 + nq - 1;                 // the tile's last query sees keys 0..last_key
     const int32_t* table = a.block_tables + (int64_t)seq * a.table_stride;
     const float slope = a.slopes ? a.slopes[head] : 0.f;
-    const TileWalk walk(a.window, a.keep_first, past + q0, AK);
+    const TileWalk walk(a.window, a.keep_first, a.chunk, past + q0, AK);
     for (int k0 = walk.first_end > 0 || walk.win_start == 0 ? 0 : walk.win_start; k0 <= last_key; k0 = walk.next(k0)) {
         __syncthreads();                                     // the previous tile's readers are done
         for (int i = tid; i < AK * dim; i += 256) {
@@ -246,7 +273,7 @@ __global__ __launch_bounds__(256) void attn_paged_any_kernel(AttnArgs a) {
             s0 = __builtin_fmaf(qv, kr0[d], s0);
             s1 = __builtin_fmaf(qv, kr1[d], s1);
         }
-        const bool ok0 = qi < nq && key_visible(k0 + sub, qpos, a.window, a.keep_first), ok1 = qi < nq && key_visible(k0 + sub + 16, qpos, a.window, a.keep_first);
+        const bool ok0 = qi < nq && key_visible(k0 + sub, qpos, a.window, a.keep_first, a.chunk), ok1 = qi < nq && key_visible(k0 + sub + 16, qpos, a.window, a.keep_first, a.chunk);
         s0 = ok0 ? s0 - slope * (float)(qpos - (k0 + sub)) : -INFINITY;
         s1 = ok1 ? s1 - slope * (float)(qpos - (k0 + sub + 16)) : -INFINITY;
         const float m_new = fmaxf(m_run, row16_max(fmaxf(s0, s1)));
@@ -390,6 +417,10 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
 #pragma unroll
     for (int i = 0; i < NVT; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
+    if (a.sinks && (!SPLIT || (wave == 0 && part == 0))) {   // the sink is what a row starts from; where waves or parts share a row, one of them holds it
+        m_run = a.sinks[head];
+        l_run = 1.f;
+    }
     const int32_t* table = a.block_tables + (int64_t)seq * a.table_stride;
     const bool wave_idle = !SPLIT && wave * 16 >= nrows;     // no row of this wave is real
     const int wave_last = SPLIT ? last_key : past + q0 + min(wave * 16 + 15, nq - 1);   // keys beyond it are masked for the whole wave
@@ -422,7 +453,7 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
     };
     // Two register sets, two tiles ahead: the loads of the tile after next are issued when a tile has been handed to LDS.
     const float slope = a.slopes ? a.slopes[head] : 0.f;
-    const TileWalk walk(a.window, a.keep_first, GROUPED ? past : past + q0, MK);
+    const TileWalk walk(a.window, a.keep_first, a.chunk, GROUPED ? past : past + q0, MK);
     bf16x8 kA[KCH], vA[VCH], kB[KCH], vB[VCH];
     // (with key parts a workgroup walks the tiles whose number is its own modulo the number of parts)
     auto mine = [&](int k0) { return nparts == 1 || (k0 / MK) % nparts == part; };
@@ -483,7 +514,7 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int key = k0 + (SPLIT ? wave : t) * 16 + fq * 4 + r;
-                const bool ok = qok && key_visible(key, qpos, a.window, a.keep_first);
+                const bool ok = qok && key_visible(key, qpos, a.window, a.keep_first, a.chunk);
                 sc[t][r] = ok ? sc[t][r] * a.scale - slope * (float)(qpos - key) : -INFINITY;
                 mx = fmaxf(mx, sc[t][r]);
             }
@@ -698,7 +729,7 @@ extern "C" int32_t nvh_attn_rotary_prep(const void* proj, int64_t proj_row_strid
                                         float eps, const int64_t* positions, const float* qk_freq, float qk_mag, int64_t rot_dims,
                                         int32_t qk_interleaved, const float* v_freq, int32_t v_interleaved, void* q_out, float* gate_out,
                                         void* k_cache, void* v_cache, const int32_t* slot_mapping, int64_t page, int64_t num_tokens,
-                                        int64_t num_q_heads, int64_t num_kv_heads, int64_t dim, int64_t vdim, int32_t act_f32,
+                                        int64_t num_q_heads, int64_t num_kv_heads, int64_t dim, int64_t vdim, int32_t norm_per_head, int32_t act_f32,
                                         nvh_stream_t stream) {
     NVH_REQUIRE(proj && positions && q_out && !q_norm_weight == !k_norm_weight, NVH_EINVAL, "nvh_attn_rotary_prep: null pointer");
     NVH_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && dim > 0 && vdim > 0 && num_tokens >= 0 && page > 0, NVH_EINVAL, "nvh_attn_rotary_prep: bad sizes");
@@ -708,11 +739,13 @@ extern "C" int32_t nvh_attn_rotary_prep(const void* proj, int64_t proj_row_strid
     NVH_REQUIRE(proj_row_stride >= (num_q_heads + num_kv_heads) * dim + num_kv_heads * vdim + (gate_out ? num_q_heads : 0), NVH_EINVAL,
                 "nvh_attn_rotary_prep: projection row too short");
     if (num_tokens == 0) return NVH_OK;
-    PrepArgs a{proj, proj_row_stride, q_norm_weight, k_norm_weight, eps, positions, qk_freq, qk_mag, (int)rot_dims, qk_interleaved,
+    PrepArgs a{proj, proj_row_stride, q_norm_weight, k_norm_weight, norm_per_head, eps, positions, qk_freq, qk_mag, (int)rot_dims, qk_interleaved,
                v_freq, v_interleaved, q_out, gate_out, k_cache, v_cache, slot_mapping, (int)num_q_heads, (int)num_kv_heads, (int)dim, (int)vdim, (int)page};
     hipStream_t st = (hipStream_t)stream;
-    if (act_f32) attn_rotary_prep_kernel<float><<<dim3((unsigned)num_tokens), 256, 0, st>>>(a);
-    else attn_rotary_prep_kernel<bf16><<<dim3((unsigned)num_tokens), 256, 0, st>>>(a);
+    const size_t lds = norm_per_head ? sizeof(float) * (size_t)(num_q_heads + num_kv_heads) : 0;
+    NVH_REQUIRE(lds <= 32 * 1024, NVH_ENOSYS, "nvh_attn_rotary_prep: %ld heads above the per-head norm's limit", (long)(num_q_heads + num_kv_heads));
+    if (act_f32) attn_rotary_prep_kernel<float><<<dim3((unsigned)num_tokens), 256, lds, st>>>(a);
+    else attn_rotary_prep_kernel<bf16><<<dim3((unsigned)num_tokens), 256, lds, st>>>(a);
     NVH_CHECK_LAUNCH("nvh_attn_rotary_prep");
     return NVH_OK;
 }
@@ -721,9 +754,10 @@ extern "C" int32_t nvh_attn_paged_any(const void* q, const void* k_cache, const 
                                       const int32_t* context_lens, const int32_t* block_tables, int64_t table_stride, int64_t batch,
                                       int64_t total_q, int64_t page, int64_t num_q_heads, int64_t num_kv_heads, int64_t dim, int64_t vdim,
                                       float scale, const float* gate, const float* v_freq, int32_t v_interleaved, const float* slopes,
-                                      int64_t window, int64_t keep_first, void* out, float* parts_ws, int64_t parts_ws_bytes, int32_t act_f32,
-                                      nvh_stream_t stream) {
+                                      int64_t window, int64_t keep_first, int64_t chunk, const float* sinks, void* out, float* parts_ws,
+                                      int64_t parts_ws_bytes, int32_t act_f32, nvh_stream_t stream) {
     NVH_REQUIRE(window >= 0 && keep_first >= 0 && window < (1 << 30) && keep_first < (1 << 30), NVH_EINVAL, "nvh_attn_paged_any: bad window");
+    NVH_REQUIRE(chunk >= 0 && chunk < (1 << 30), NVH_EINVAL, "nvh_attn_paged_any: bad chunk");
     NVH_REQUIRE(q && k_cache && v_cache && context_lens && block_tables && out, NVH_EINVAL, "nvh_attn_paged_any: null pointer");
     NVH_REQUIRE(batch >= 0 && total_q >= 0 && page > 0 && num_q_heads > 0 && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0 && dim > 0 && vdim > 0,
                 NVH_EINVAL, "nvh_attn_paged_any: bad sizes");
@@ -740,7 +774,7 @@ extern "C" int32_t nvh_attn_paged_any(const void* q, const void* k_cache, const 
     }
     if (batch == 0 || total_q == 0) return NVH_OK;
     AttnArgs a{q, k_cache, v_cache, cu_seqlens_q, context_lens, block_tables, table_stride, (int)batch, (int)page, (int)num_q_heads,
-               (int)num_kv_heads, (int)dim, (int)vdim, scale, gate, v_freq, v_interleaved, out, slopes, (int)window, (int)keep_first, 0, 0, 1, 1, nullptr};
+               (int)num_kv_heads, (int)dim, (int)vdim, scale, gate, v_freq, v_interleaved, out, slopes, (int)window, (int)keep_first, (int)chunk, sinks, 0, 0, 1, 1, nullptr};
     // at most ceil(len / AQ) tiles per sequence: total_q / AQ + batch bounds their number (surplus workgroups exit)
     const dim3 grid((unsigned)(total_q / AQ + batch), (unsigned)num_q_heads);
     hipStream_t st = (hipStream_t)stream;

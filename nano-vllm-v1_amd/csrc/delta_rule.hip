@@ -11,6 +11,13 @@
 //                    of 16), each with every 16th (4th) row, which meet twice per token in a cross-lane sum.  The order of every sum is fixed by the sizes alone: decoding
 //                    token by token, in portions or in one piece gives the same bits.
 //   nvh_delta_post   per head: o / rms(o), times the norm weight and the sigmoid output gate, to the activation type.
+//   nvh_gated_delta_prep   the gated delta rule, S <- g S; d = beta (v - S^T k); S <- S + k d^T; o = S^T q, with one decay g per head
+//                    and a write strength beta per head, is the recurrence above with w = g on every channel, u = k (a unit
+//                    vector), a u = beta g k and the written key beta k: g S - beta g k (k^T S) + beta k v^T.  The prep runs the
+//                    short causal convolution (continued from the sequence's carried inputs) and silu over the q | k | v
+//                    channels, makes q and k unit vectors per head (q also times dk^-1/2), forms beta = sigmoid(b) and
+//                    g = exp(-exp(A_log) softplus(a + dt_bias)), all in fp32, and leaves the scan's rows; q and k heads
+//                    may be shared by groups of value heads, and the value size is free.
 #include "common.h"
 
 namespace {
@@ -33,6 +40,93 @@ struct DeltaPrepArgs {
     int H, dk, rank;
     float decay_scale;
 };
+
+struct GatedDeltaPrepArgs {
+    const void* qkv;           // [T, ld]: the convolved channels q (G dk) | k (G dk) | v (H dv) of the projection row
+    int64_t qkv_stride;
+    const void *b, *a;         // [T, ld]: H columns each (write strength and decay logits)
+    int64_t b_stride, a_stride;
+    const void* conv_w;        // [C, taps], last column on the current token
+    const void *dt_bias, *a_log;    // [H]
+    const float* conv_state;   // [slots, taps - 1, C]
+    const int32_t *slots, *cu_seqlens_q, *context_lens;
+    float* out;                // [T, H, 5 dk + dv]: q | beta k | g | k | beta g k | v
+    int batch, taps, H, G, dk, dv;
+};
+
+__device__ __forceinline__ float softplusf_(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+
+// One workgroup per token.  The convolved, activated channels meet in LDS; a wave per q / k head sums its squares; then every
+// head's row is written.
+template <typename A>
+__global__ __launch_bounds__(256) void gated_delta_prep_kernel(GatedDeltaPrepArgs p) {
+    extern __shared__ float sh[];                            // [C] channels, then [2 G] inverse lengths, then [H] beta, [H] g
+    const int64_t t = blockIdx.x;
+    const int nqk = p.G * p.dk, C = 2 * nqk + p.H * p.dv, taps = p.taps;
+    float* inv = sh + C;
+    float* beta = inv + 2 * p.G;
+    float* dec = beta + p.H;
+    int seq = 0;
+    if (p.cu_seqlens_q) {
+        int lo_b = 0, hi_b = p.batch;                        // the sequence whose rows hold token t
+        while (hi_b - lo_b > 1) {
+            const int mid = (lo_b + hi_b) >> 1;
+            if (p.cu_seqlens_q[mid] <= t) lo_b = mid; else hi_b = mid;
+        }
+        seq = lo_b;
+    } else {
+        seq = (int)t;
+    }
+    const int lo = p.cu_seqlens_q ? p.cu_seqlens_q[seq] : seq, hi = p.cu_seqlens_q ? p.cu_seqlens_q[seq + 1] : seq + 1;
+    const int j = (int)t - lo;
+    const int slot = p.slots[seq];
+    const bool carried = slot >= 0 && p.context_lens[seq] != hi - lo;
+    const float* st = carried ? p.conv_state + (int64_t)slot * (taps - 1) * C : nullptr;
+    for (int c = threadIdx.x; c < C; c += 256) {
+        float acc = 0.f;
+        for (int k = 0; k < taps; ++k) {                     // tap k multiplies the input taps - 1 - k tokens back
+            const int back = taps - 1 - k, src = j - back;
+            float in = 0.f;
+            if (src >= 0) in = ldf((const A*)p.qkv, (t - back) * p.qkv_stride + c);
+            else if (st) in = st[(int64_t)(taps - 1 + src) * C + c];
+            acc = __builtin_fmaf(ldf((const A*)p.conv_w, (int64_t)c * taps + k), in, acc);
+        }
+        sh[c] = acc / (1.0f + expf(-acc));
+    }
+    for (int h = threadIdx.x; h < p.H; h += 256) {
+        beta[h] = sigmoidf_(ldf((const A*)p.b, t * p.b_stride + h));
+        const float dt = softplusf_(ldf((const A*)p.a, t * p.a_stride + h) + ldf((const A*)p.dt_bias, h));
+        dec[h] = expf(-expf(ldf((const A*)p.a_log, h)) * dt);
+    }
+    __syncthreads();
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int g = wave; g < 2 * p.G; g += 4) {                // q heads, then k heads (they lie one after the other)
+        float ss = 0.f;
+        for (int i = lane; i < p.dk; i += 64) ss += sh[g * p.dk + i] * sh[g * p.dk + i];
+        ss = wave_sum(ss);
+        if (lane == 0) inv[g] = 1.0f / sqrtf(ss + 1e-6f);
+    }
+    __syncthreads();
+    const int dk = p.dk, dv = p.dv, row = 5 * dk + dv, per = p.H / p.G;
+    const float qs = 1.0f / sqrtf((float)dk);
+    float* out = p.out + t * (int64_t)p.H * row;
+    for (int e = threadIdx.x; e < p.H * row; e += 256) {
+        const int h = e / row, r = e - h * row, g = h / per;
+        float v;
+        if (r >= 5 * dk) {
+            v = sh[2 * nqk + h * dv + (r - 5 * dk)];
+        } else {
+            const int part = r / dk, i = r - part * dk;
+            const float ku = sh[nqk + g * dk + i] * inv[p.G + g];
+            if (part == 0) v = sh[g * dk + i] * inv[g] * qs;
+            else if (part == 1) v = beta[h] * ku;
+            else if (part == 2) v = dec[h];
+            else if (part == 3) v = ku;
+            else v = beta[h] * dec[h] * ku;
+        }
+        out[e] = v;
+    }
+}
 
 template <typename A>
 __global__ __launch_bounds__(256) void delta_prep_kernel(DeltaPrepArgs p) {
@@ -69,12 +163,12 @@ __global__ __launch_bounds__(256) void delta_prep_kernel(DeltaPrepArgs p) {
 }
 
 struct DeltaScanArgs {
-    const float* pack;         // [T, H, 6, dk] from delta_prep_kernel
-    float* state;              // [slots, H, dk, dk]
+    const float* pack;         // [T, H, 5 dk + dv]: r | k | w | u | a*u (dk each) | v (dv) per head, from a prep kernel
+    float* state;              // [slots, H, dk, dv]
     const int32_t* slots;      // [B]
     const int32_t* cu_seqlens_q;    // [B+1] or null (one token per sequence)
     const int32_t* context_lens;    // [B]: tokens of the sequence including this step's (a step that holds them all starts from zero)
-    float* out;                // [T, H*dk]
+    float* out;                // [T, H*dv]
     int H, dk, dv;
 };
 
@@ -107,8 +201,9 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaScanArgs p) {
     // Row of a token as this workgroup needs it: the five dk-vectors, then its COLS columns of v.  Every load is
     // unconditional (indices clamped into the row and into the sequence), so all of a stage's loads are in flight together.
     float pre[TOK][CH];
-    const float* base = p.pack + (int64_t)head * 6 * dk;
-    const int64_t tok_stride = (int64_t)p.H * 6 * dk;
+    const int prow = 5 * dk + dv;                            // a head's row of the pack
+    const float* base = p.pack + (int64_t)head * prow;
+    const int64_t tok_stride = (int64_t)p.H * prow;
     auto fetch = [&](int t0) {
 #pragma unroll
         for (int tt = 0; tt < TOK; ++tt) {
@@ -116,7 +211,7 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaScanArgs p) {
 #pragma unroll
             for (int c = 0; c < CH; ++c) {
                 const int e = threadIdx.x + 256 * c;
-                const int src = min(e < 5 * dk ? e : e + col0, 6 * dk - 1);
+                const int src = min(e < 5 * dk ? e : e + col0, prow - 1);
                 pre[tt][c] = base[tok * tok_stride + src];
             }
         }
@@ -292,13 +387,36 @@ static int32_t launch_delta_scan(const DeltaScanArgs& p, int64_t batch, hipStrea
     return NVH_OK;
 }
 
+extern "C" int32_t nvh_gated_delta_prep(const void* qkv, int64_t qkv_stride, const void* b, int64_t b_stride, const void* a, int64_t a_stride,
+                                        const void* conv_w, const void* dt_bias, const void* a_log, const float* conv_state, const int32_t* slots,
+                                        const int32_t* cu_seqlens_q, const int32_t* context_lens, float* out, int64_t batch, int64_t num_tokens,
+                                        int64_t taps, int64_t heads, int64_t qk_heads, int64_t dk, int64_t dv, int32_t act_f32, nvh_stream_t stream) {
+    NVH_REQUIRE(qkv && b && a && conv_w && dt_bias && a_log && slots && context_lens && out, NVH_EINVAL, "nvh_gated_delta_prep: null pointer");
+    NVH_REQUIRE(batch >= 0 && num_tokens >= 0 && taps >= 1 && heads > 0 && qk_heads > 0 && heads % qk_heads == 0 && dk > 0 && dv > 0, NVH_EINVAL,
+                "nvh_gated_delta_prep: bad sizes");
+    NVH_REQUIRE(taps == 1 || conv_state, NVH_EINVAL, "nvh_gated_delta_prep: null state");
+    NVH_REQUIRE(cu_seqlens_q || num_tokens == batch, NVH_EINVAL, "nvh_gated_delta_prep: one token per sequence without cu_seqlens_q");
+    const int64_t channels = 2 * qk_heads * dk + heads * dv;
+    NVH_REQUIRE(qkv_stride >= channels, NVH_EINVAL, "nvh_gated_delta_prep: projection row too short");
+    const size_t lds = sizeof(float) * (size_t)(channels + 2 * qk_heads + 2 * heads);
+    NVH_REQUIRE(lds <= 64 * 1024, NVH_ENOSYS, "nvh_gated_delta_prep: %ld channels above the kernel's limit", (long)channels);
+    if (num_tokens == 0 || batch == 0) return NVH_OK;
+    GatedDeltaPrepArgs p{qkv, qkv_stride, b, a, b_stride, a_stride, conv_w, dt_bias, a_log, conv_state, slots, cu_seqlens_q, context_lens, out,
+                         (int)batch, (int)taps, (int)heads, (int)qk_heads, (int)dk, (int)dv};
+    hipStream_t st = (hipStream_t)stream;
+    if (act_f32) gated_delta_prep_kernel<float><<<dim3((unsigned)num_tokens), 256, lds, st>>>(p);
+    else gated_delta_prep_kernel<bf16><<<dim3((unsigned)num_tokens), 256, lds, st>>>(p);
+    NVH_CHECK_LAUNCH("nvh_gated_delta_prep");
+    return NVH_OK;
+}
+
 extern "C" int32_t nvh_delta_scan(const float* pack, float* state, const int32_t* slots, const int32_t* cu_seqlens_q,
-                                  const int32_t* context_lens, float* out, int64_t batch, int64_t heads, int64_t dk, nvh_stream_t stream) {
+                                  const int32_t* context_lens, float* out, int64_t batch, int64_t heads, int64_t dk, int64_t dv, nvh_stream_t stream) {
     NVH_REQUIRE(pack && state && slots && context_lens && out, NVH_EINVAL, "nvh_delta_scan: null pointer");
-    NVH_REQUIRE(batch >= 0 && heads > 0 && dk > 0, NVH_EINVAL, "nvh_delta_scan: bad sizes");
+    NVH_REQUIRE(batch >= 0 && heads > 0 && dk > 0 && dv > 0, NVH_EINVAL, "nvh_delta_scan: bad sizes");
     NVH_REQUIRE(dk <= 256, NVH_ENOSYS, "nvh_delta_scan: key size %ld above 256", (long)dk);
     if (batch == 0) return NVH_OK;
-    DeltaScanArgs p{pack, state, slots, cu_seqlens_q, context_lens, out, (int)heads, (int)dk, (int)dk};
+    DeltaScanArgs p{pack, state, slots, cu_seqlens_q, context_lens, out, (int)heads, (int)dk, (int)dv};
     return launch_delta_scan(p, batch, (hipStream_t)stream);
 }
 

@@ -352,6 +352,44 @@ __global__ __launch_bounds__(256) void conv_state_update_kernel(SsdPrepArgs p) {
     }
 }
 
+// The residual stream plus its own short causal convolution over time, per column: h_t = x_t + sum_k w[:, k] x_(t - taps + 1 + k), the
+// last tap on the token itself, zeros before the sequence's start, continued across steps from the sequence's carried rows
+// (state [slots, taps - 1, dim], brought up to date by nvh_conv_state_update afterwards).  x and the sums are fp32; h leaves in
+// the activation type.  One workgroup per token.
+struct StreamConvArgs {
+    const float* x;            // [T, dim]
+    const void* w;             // [dim, taps]
+    const float* state;
+    const int32_t *slots, *cu_seqlens_q, *context_lens;
+    void* h;
+    int64_t h_stride;
+    int batch, taps, dim;
+};
+
+template <typename A>
+__global__ __launch_bounds__(256) void stream_conv_kernel(StreamConvArgs p) {
+    const int64_t t = blockIdx.x;
+    const int seq = seq_of_token(p.cu_seqlens_q, p.batch, t);
+    const int lo = p.cu_seqlens_q ? p.cu_seqlens_q[seq] : seq, hi = p.cu_seqlens_q ? p.cu_seqlens_q[seq + 1] : seq + 1;
+    const int j = (int)t - lo, taps = p.taps, dim = p.dim;
+    const int slot = p.slots[seq];
+    const bool carried = slot >= 0 && p.context_lens[seq] != hi - lo;
+    const float* st = carried ? p.state + (int64_t)slot * (taps - 1) * dim : nullptr;
+    A* h = (A*)p.h + t * p.h_stride;
+    for (int c = blockIdx.y * 256 + threadIdx.x; c < dim; c += 256 * gridDim.y) {
+        const float cur = p.x[t * dim + c];
+        float acc = 0.f;
+        for (int k = 0; k < taps; ++k) {
+            const int back = taps - 1 - k, src = j - back;
+            float in = 0.f;
+            if (src >= 0) in = p.x[(t - back) * dim + c];
+            else if (st) in = st[(int64_t)(taps - 1 + src) * dim + c];
+            acc = __builtin_fmaf(ldf((const A*)p.w, (int64_t)c * taps + k), in, acc);
+        }
+        h[c] = (A)(cur + acc);
+    }
+}
+
 // ---------------------------------------------------------------------------------------------------------------
 struct ScanArgs {
     const float *q, *k;        // [T, QG, dk]: head h reads group h / (H / QG)
@@ -826,6 +864,23 @@ extern "C" int32_t nvh_conv_state_update(const void* xbc, int64_t xbc_stride, fl
     if (act_f32) conv_state_update_kernel<float><<<grid, 256, 0, st>>>(p);
     else conv_state_update_kernel<bf16><<<grid, 256, 0, st>>>(p);
     NVH_CHECK_LAUNCH("nvh_conv_state_update");
+    return NVH_OK;
+}
+
+extern "C" int32_t nvh_stream_conv(const float* x, const void* w, const float* state, const int32_t* slots, const int32_t* cu_seqlens_q,
+                                   const int32_t* context_lens, void* h, int64_t h_stride, int64_t batch, int64_t num_tokens, int64_t taps, int64_t dim,
+                                   int32_t act_f32, nvh_stream_t stream) {
+    NVH_REQUIRE(x && w && slots && context_lens && h && batch >= 0 && num_tokens >= 0 && taps >= 1 && dim > 0 && h_stride >= dim, NVH_EINVAL,
+                "nvh_stream_conv: bad argument");
+    NVH_REQUIRE(taps == 1 || state, NVH_EINVAL, "nvh_stream_conv: null state");
+    NVH_REQUIRE(cu_seqlens_q || num_tokens == batch, NVH_EINVAL, "nvh_stream_conv: one token per sequence without cu_seqlens_q");
+    if (num_tokens == 0 || batch == 0) return NVH_OK;
+    const StreamConvArgs p{x, w, state, slots, cu_seqlens_q, context_lens, h, h_stride, (int)batch, (int)taps, (int)dim};
+    hipStream_t st = (hipStream_t)stream;
+    const dim3 grid((unsigned)num_tokens, (unsigned)(num_tokens >= 512 ? 1 : std::min<int64_t>(nvh_cdiv(dim, 256), 16)));
+    if (act_f32) stream_conv_kernel<float><<<grid, 256, 0, st>>>(p);
+    else stream_conv_kernel<bf16><<<grid, 256, 0, st>>>(p);
+    NVH_CHECK_LAUNCH("nvh_stream_conv");
     return NVH_OK;
 }
 

@@ -72,7 +72,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
 template <typename A>
 __global__ __launch_bounds__(256) void moe_route_linear_kernel(const A* __restrict__ x, int64_t ldx, const A* __restrict__ w, const A* __restrict__ bias,
                                                                int32_t* __restrict__ ids, float* __restrict__ weights, float* __restrict__ logits_out,
-                                                               int experts, int K, int top, int vec) {
+                                                               int experts, int K, int top, int vec, int sigmoid_scores) {
     __shared__ float zs[64 * ROUTE_MAX_PER_LANE];
     const int64_t t = blockIdx.x;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -130,7 +130,8 @@ __global__ __launch_bounds__(256) void moe_route_linear_kernel(const A* __restri
             }
         }
         if (r == 0) first = bv;
-        const float wgt = expf(bv - first);
+        // (sigmoid scores: an expert's weight is its own score, whatever the others'; the order by logit is the order by score)
+        const float wgt = sigmoid_scores ? 1.0f / (1.0f + expf(-bv)) : expf(bv - first);
         denom += wgt;
         if (lane == 0) {
             ids[t * top + r] = be;
@@ -140,7 +141,7 @@ __global__ __launch_bounds__(256) void moe_route_linear_kernel(const A* __restri
         for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j)
             if (lane + 64 * j == be) z[j] = -INFINITY;
     }
-    if (lane == 0)
+    if (lane == 0 && !sigmoid_scores)
         for (int r = 0; r < top; ++r) weights[t * top + r] = weights[t * top + r] / denom;
 }
 
@@ -400,10 +401,31 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const A* __restrict__ 
         float s = 0.f;
         for (int r = 0; r < top; ++r) {
             const int pos = pos_of_pair[t * top + r];
-            if (pos >= 0) s = __builtin_fmaf(weights[t * top + r], (float)y[(int64_t)pos * ldy + c], s);
+            if (pos >= 0) s = __builtin_fmaf(weights ? weights[t * top + r] : 1.0f, (float)y[(int64_t)pos * ldy + c], s);
         }
         if (shared) s += sg * (float)shared[t * shared_stride + c];
         out[t * dim + c] = s;
+    }
+}
+
+// The experts' activation where a pair's routing weight multiplies the expert's INPUT: the rows of the first grouped product were
+// formed from the unweighted token, and since that product is linear, row * weight is the product of the weighted token.  Then, with
+// the gate's value capped above and the other half's value clamped to +-limit,
+//   g = min(w G, limit);  u = clamp(w U, -limit, limit);  y = g sigmoid(alpha g) (u + 1).
+// One workgroup per (token, choice) pair; its row is pos_of_pair[pair] (< 0: the pair has no row).
+template <typename A>
+__global__ __launch_bounds__(256) void glu_clamp_pairs_kernel(const A* __restrict__ gu, int64_t gu_stride, const int32_t* __restrict__ pos_of_pair,
+                                                              const float* __restrict__ weights, A* __restrict__ y, int64_t y_stride, int inter, float limit,
+                                                              float alpha) {
+    const int64_t pair = blockIdx.x;
+    const int pos = pos_of_pair[pair];
+    if (pos < 0) return;
+    const float w = weights ? weights[pair] : 1.0f;
+    const A* row = gu + (int64_t)pos * gu_stride;
+    for (int c = threadIdx.x; c < inter; c += 256) {
+        const float g = fminf((float)row[c] * w, limit);
+        const float u = fminf(fmaxf((float)row[inter + c] * w, -limit), limit);
+        y[(int64_t)pos * y_stride + c] = (A)(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
     }
 }
 
@@ -421,8 +443,8 @@ extern "C" int32_t nvh_moe_route(const float* logits, int64_t row_stride, int32_
 }
 
 extern "C" int32_t nvh_moe_route_linear(const void* x, int64_t x_row_stride, const void* w, const void* bias, int32_t* ids, float* weights,
-                                        float* logits_out, int64_t num_tokens, int64_t experts, int64_t K, int64_t top, int32_t act_f32,
-                                        nvh_stream_t stream) {
+                                        float* logits_out, int64_t num_tokens, int64_t experts, int64_t K, int64_t top, int32_t sigmoid_scores,
+                                        int32_t act_f32, nvh_stream_t stream) {
     NVH_REQUIRE(x && w && ids && weights, NVH_EINVAL, "nvh_moe_route_linear: null pointer");
     NVH_REQUIRE(num_tokens >= 0 && experts > 0 && top > 0 && top <= experts && K > 0 && K < (1 << 30) && x_row_stride >= K, NVH_EINVAL, "nvh_moe_route_linear: bad sizes");
     NVH_REQUIRE(experts <= 64 * ROUTE_MAX_PER_LANE, NVH_ENOSYS, "nvh_moe_route_linear: %ld experts above %d", (long)experts, 64 * ROUTE_MAX_PER_LANE);
@@ -430,8 +452,8 @@ extern "C" int32_t nvh_moe_route_linear(const void* x, int64_t x_row_stride, con
     const dim3 grid((unsigned)num_tokens);
     hipStream_t st = (hipStream_t)stream;
     const int vec = K % 8 == 0 && x_row_stride % 8 == 0 && nvh_aligned16(x) && nvh_aligned16(w);
-    if (act_f32) moe_route_linear_kernel<float><<<grid, 256, 0, st>>>((const float*)x, x_row_stride, (const float*)w, (const float*)bias, ids, weights, logits_out, (int)experts, (int)K, (int)top, vec);
-    else moe_route_linear_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)x, x_row_stride, (const bf16*)w, (const bf16*)bias, ids, weights, logits_out, (int)experts, (int)K, (int)top, vec);
+    if (act_f32) moe_route_linear_kernel<float><<<grid, 256, 0, st>>>((const float*)x, x_row_stride, (const float*)w, (const float*)bias, ids, weights, logits_out, (int)experts, (int)K, (int)top, vec, sigmoid_scores);
+    else moe_route_linear_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)x, x_row_stride, (const bf16*)w, (const bf16*)bias, ids, weights, logits_out, (int)experts, (int)K, (int)top, vec, sigmoid_scores);
     NVH_CHECK_LAUNCH("nvh_moe_route_linear");
     return NVH_OK;
 }
@@ -499,10 +521,22 @@ extern "C" int32_t nvh_gemm_grouped_any_nt(const void* x, int64_t x_row_stride, 
     return NVH_OK;
 }
 
+extern "C" int32_t nvh_glu_clamp_pairs(const void* gate_up, int64_t row_stride, const int32_t* pos_of_pair, const float* weights, void* y, int64_t y_stride,
+                                       int64_t pairs, int64_t inter, float limit, float alpha, int32_t act_f32, nvh_stream_t stream) {
+    NVH_REQUIRE(gate_up && pos_of_pair && y && pairs >= 0 && inter > 0 && row_stride >= 2 * inter && y_stride >= inter && limit > 0.f, NVH_EINVAL,
+                "nvh_glu_clamp_pairs: bad argument");
+    if (pairs == 0) return NVH_OK;
+    hipStream_t st = (hipStream_t)stream;
+    if (act_f32) glu_clamp_pairs_kernel<float><<<dim3((unsigned)pairs), 256, 0, st>>>((const float*)gate_up, row_stride, pos_of_pair, weights, (float*)y, y_stride, (int)inter, limit, alpha);
+    else glu_clamp_pairs_kernel<bf16><<<dim3((unsigned)pairs), 256, 0, st>>>((const bf16*)gate_up, row_stride, pos_of_pair, weights, (bf16*)y, y_stride, (int)inter, limit, alpha);
+    NVH_CHECK_LAUNCH("nvh_glu_clamp_pairs");
+    return NVH_OK;
+}
+
 extern "C" int32_t nvh_moe_combine(const void* y, int64_t y_row_stride, const int32_t* pos_of_pair, const float* weights, const void* shared,
                                    int64_t shared_stride, const float* shared_gate, int64_t shared_gate_stride, float* out, int64_t num_tokens, int64_t dim,
                                    int64_t top, int32_t act_f32, nvh_stream_t stream) {
-    NVH_REQUIRE(y && pos_of_pair && weights && out && num_tokens >= 0 && dim > 0 && top > 0 && y_row_stride >= dim, NVH_EINVAL, "nvh_moe_combine: bad argument");
+    NVH_REQUIRE(y && pos_of_pair && out && num_tokens >= 0 && dim > 0 && top > 0 && y_row_stride >= dim, NVH_EINVAL, "nvh_moe_combine: bad argument");
     if (num_tokens == 0) return NVH_OK;
     hipStream_t st = (hipStream_t)stream;
     if (act_f32) moe_combine_kernel<float><<<dim3((unsigned)num_tokens), 256, 0, st>>>((const float*)y, y_row_stride, pos_of_pair, weights, (const float*)shared, shared_stride, shared_gate, shared_gate_stride, out, (int)dim, (int)top);

@@ -286,6 +286,52 @@ __global__ __launch_bounds__(256) void residual_postnorm_kernel(PostNormArgs p) 
     }
 }
 
+// The close of a sublayer whose RESULT is normed before it joins the stream (the sublayer itself read the stream as it is), per row:
+//   y = sa a + sb b + c32;   x <- x + mult * w * y / sqrt(mean(y^2) + eps);   h <- x in the activation type (when asked for)
+// a, b (type A) and c32 (fp32) are the sublayer's terms, any of them absent; w: one number for all columns (w_elems 1) or one a
+// column.  Sums, statistics and the stream are fp32; the row sits in LDS between the two passes.
+struct SubNormArgs {
+    const void *a, *b;
+    const float* c32;
+    int64_t a_stride, b_stride, c32_stride;
+    float sa, sb, mult, eps;
+    const void* w;
+    int w_elems;
+    float* x;
+    void* h;
+    int64_t h_stride;
+    int dim;
+};
+
+template <typename A>
+__global__ __launch_bounds__(256) void residual_subnorm_kernel(SubNormArgs p) {
+    extern __shared__ float rowbuf[];
+    __shared__ float red[4];
+    const int64_t row = blockIdx.x;
+    const int dim = p.dim;
+    const A* a = p.a ? (const A*)p.a + row * p.a_stride : nullptr;
+    const A* b = p.b ? (const A*)p.b + row * p.b_stride : nullptr;
+    const float* c32 = p.c32 ? p.c32 + row * p.c32_stride : nullptr;
+    float sq = 0.f;
+    for (int i = threadIdx.x; i < dim; i += 256) {
+        float y = 0.f;
+        if (a) y = p.sa * (float)a[i];
+        if (b) y = __builtin_fmaf(p.sb, (float)b[i], y);
+        if (c32) y += c32[i];
+        rowbuf[i] = y;
+        sq += y * y;
+    }
+    const float inv = p.mult / sqrtf(block_sum4(sq, red) / (float)dim + p.eps);
+    float* xr = p.x + row * dim;
+    A* h = p.h ? (A*)p.h + row * p.h_stride : nullptr;
+    const A* w = (const A*)p.w;
+    for (int i = threadIdx.x; i < dim; i += 256) {
+        const float v = xr[i] + rowbuf[i] * inv * (float)w[p.w_elems == 1 ? 0 : i];
+        xr[i] = v;
+        if (h) h[i] = (A)v;
+    }
+}
+
 // y = act(g) (* u when gated): g = columns [0, inter) and u = columns [inter, 2 inter) of the row.
 // act: 0 silu, 1 gelu (tanh form), 2 squared relu.
 template <typename A>
@@ -483,6 +529,25 @@ extern "C" int32_t nvh_residual_postnorm(const void* y, int64_t y_stride, const 
     if (act_f32) residual_postnorm_kernel<float><<<dim3((unsigned)rows), 256, lds, st>>>(p);
     else residual_postnorm_kernel<bf16><<<dim3((unsigned)rows), 256, lds, st>>>(p);
     NVH_CHECK_LAUNCH("nvh_residual_postnorm");
+    return NVH_OK;
+}
+
+extern "C" int32_t nvh_residual_subnorm(const void* a, int64_t a_stride, float a_scale, const void* b, int64_t b_stride, float b_scale, const float* c32,
+                                        int64_t c32_stride, float mult, const void* weight, int64_t weight_elems, float eps, float* x, void* h,
+                                        int64_t h_stride, int64_t rows, int64_t dim, int32_t act_f32, nvh_stream_t stream) {
+    NVH_STREAM_ARGS_OK("nvh_residual_subnorm", x && weight && (a || b || c32) && rows >= 0 && dim > 0 && dim <= 32768 && (weight_elems == 1 || weight_elems == dim));
+    if (rows == 0) return NVH_OK;
+    const SubNormArgs p{a, b, c32, a_stride, b_stride, c32_stride, a_scale, b_scale, mult, eps, weight, (int)weight_elems, x, h, h_stride, (int)dim};
+    hipStream_t st = (hipStream_t)stream;
+    const size_t lds = sizeof(float) * (size_t)dim;
+    if (lds > 48 * 1024) {
+        const hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(&residual_subnorm_kernel<float>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        const hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(&residual_subnorm_kernel<bf16>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        NVH_REQUIRE(e1 == hipSuccess && e2 == hipSuccess, NVH_ENOSYS, "nvh_residual_subnorm: %zu bytes of LDS refused", lds);
+    }
+    if (act_f32) residual_subnorm_kernel<float><<<dim3((unsigned)rows), 256, lds, st>>>(p);
+    else residual_subnorm_kernel<bf16><<<dim3((unsigned)rows), 256, lds, st>>>(p);
+    NVH_CHECK_LAUNCH("nvh_residual_subnorm");
     return NVH_OK;
 }
 

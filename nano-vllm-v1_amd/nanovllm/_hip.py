@@ -97,16 +97,18 @@ SIGNATURES = {
     "nvh_gather_rows_f32": (i32, [vp, vp, vp, i64, i64, vp]),
     "nvh_logit_softcap": (i32, [vp, i64, vp, i64, i64, f32, i32, vp]),
     "nvh_gemm_any_nt": (i32, [vp, i64, vp, vp, vp, i64, i64, i64, i64, i32, i32, vp]),
-    "nvh_attn_rotary_prep": (i32, [vp, i64, vp, vp, f32, vp, vp, f32, i64, i32, vp, i32, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i32, vp]),
-    "nvh_attn_paged_any": (i32, [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64, f32, vp, vp, i32, vp, i64, i64, vp, vp, i64, i32, vp]),
+    "nvh_attn_rotary_prep": (i32, [vp, i64, vp, vp, f32, vp, vp, f32, i64, i32, vp, i32, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i32, i32, vp]),
+    "nvh_attn_paged_any": (i32, [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64, f32, vp, vp, i32, vp, i64, i64, i64, vp, vp, vp, i64, i32, vp]),
     "nvh_attn_paged_any_parts_bytes": (i64, [i64, i64, i64, i64, i64, i64, i64, i32, i32]),
     "nvh_delta_prep": (i32, [vp, i64, vp, i64, vp, i64, vp, i64, vp, i64, vp, vp, vp, vp, i64, i64, i64, i64, f32, i32, vp]),
-    "nvh_delta_scan": (i32, [vp, vp, vp, vp, vp, vp, i64, i64, i64, vp]),
+    "nvh_delta_scan": (i32, [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, vp]),
+    "nvh_gated_delta_prep": (i32, [vp, i64, vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i32, vp]),
     "nvh_delta_post": (i32, [vp, vp, vp, i64, vp, i64, i64, i64, i64, f32, i32, vp]),
     # layer norm / RMS norm around the fp32 stream, plain activations (csrc/stream_f32.hip)
     "nvh_embedding_pos_stream": (i32, [vp, vp, vp, vp, f32, vp, i64, i64, i64, i64, i32, vp]),
     "nvh_residual_norm": (i32, [vp, i64, vp, vp, i64, vp, f32, f32, vp, i64, vp, i64, vp, i32, vp, vp, f32, vp, i64, i64, i64, i32, vp]),
     "nvh_residual_postnorm": (i32, [vp, i64, vp, i64, vp, f32, vp, i32, vp, f32, f32, vp, i64, i64, i64, i32, vp]),
+    "nvh_residual_subnorm": (i32, [vp, i64, f32, vp, i64, f32, vp, i64, f32, vp, i64, f32, vp, vp, i64, i64, i64, i32, vp]),
     "nvh_act_mul": (i32, [vp, i64, vp, i64, i64, i64, i32, i32, i32, vp]),
     "nvh_logits_scale": (i32, [vp, i64, vp, i64, i64, f32, f32, i32, vp]),
     # linear recurrences with a diagonal decay (csrc/linear_recurrence.hip)
@@ -119,10 +121,12 @@ SIGNATURES = {
     "nvh_rotary_qkv_prep": (i32, [vp, i64, vp, i64, vp, i64, vp, vp, f32, i64, i32, f32, f32, vp, vp, vp, i64, i64, i64, i64, i32, vp]),
     "nvh_ssd_conv_prep": (i32, [vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, vp, vp, vp, vp, i32, vp]),
     "nvh_conv_state_update": (i32, [vp, i64, vp, vp, vp, vp, i64, i64, i64, i32, vp]),
+    "nvh_stream_conv": (i32, [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp]),
     "nvh_group_rmsnorm_gate": (i32, [vp, vp, i32, vp, i64, i32, i32, vp, i64, i64, i64, i64, f32, i32, vp]),
     # mixture of experts (csrc/moe.hip)
     "nvh_moe_route": (i32, [vp, i64, vp, vp, i64, i64, i64, vp]),
-    "nvh_moe_route_linear": (i32, [vp, i64, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp]),
+    "nvh_moe_route_linear": (i32, [vp, i64, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, i32, vp]),
+    "nvh_glu_clamp_pairs": (i32, [vp, i64, vp, vp, vp, i64, i64, i64, f32, f32, i32, vp]),
     "nvh_moe_max_tiles": (i64, [i64, i64]),
     "nvh_moe_align": (i32, [vp, i64, i64, i64, vp, vp, vp, vp, vp, i64, vp]),
     "nvh_gemm_grouped_any_nt": (i32, [vp, i64, vp, vp, vp, i64, vp, vp, vp, i64, i64, i64, i32, i32, vp]),

@@ -71,21 +71,30 @@ class GatedValueRotaryAttention(nn.Module):
     cached (each head's output is turned back by the query's position), and optionally a per-head sigmoid output gate.
 
     Input is the fused projection output [T, H*dim + G*dim + G*vdim (+ H)] = q | k | v | gate; RMS norms over the WHOLE
-    q and k projections run with the rotary in one launch (nvh_attn_rotary_prep), attention in a second
-    (nvh_attn_paged_any).  A module that serves several passes of a looped stack owns one cache per pass:
+    q and k projections (or, with `norm_per_head`, over every head by itself with a weight row [dim] that the heads share) run
+    with the rotary in one launch (nvh_attn_rotary_prep), attention in a second (nvh_attn_paged_any).  `chunk` > 0: a query
+    sees only the earlier tokens of its own block of `chunk` positions, blocks counted from the sequence's start.  `sinks`: a
+    learned logit per head (parameter `sinks`, fp32) joins the softmax's denominator once - it has no key and no value and is
+    not multiplied by `scale` - so a head can give weight to nothing.  A module that serves several passes of a looped stack
+    owns one cache per pass:
     `k_caches[run]` [pages, page, G, dim] and `v_caches[run]` [pages, G, vdim, page] (values lie transposed within a page),
     bound by the runner (`cache_runs` of each)."""
 
     def __init__(self, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, scale: float, eps: float,
-                 rot_dims: int, qk_freq: torch.Tensor, qk_mag: float, value_freq: torch.Tensor | None, gated: bool,
-                 cache_runs: int = 1, interleaved: bool = False):
+                 rot_dims: int, qk_freq: torch.Tensor | None, qk_mag: float, value_freq: torch.Tensor | None, gated: bool,
+                 cache_runs: int = 1, interleaved: bool = False, norm_per_head: bool = False, chunk: int = 0, sinks: bool = False):
         super().__init__()
-        assert num_heads % num_kv_heads == 0
+        assert num_heads % num_kv_heads == 0 and chunk >= 0 and (rot_dims == 0 or qk_freq is not None)
         self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim = num_heads, num_kv_heads, head_dim, value_dim
         self.scale, self.eps, self.rot_dims, self.qk_mag, self.gated, self.interleaved = scale, eps, rot_dims, qk_mag, gated, interleaved
-        self.q_norm = nn.Parameter(torch.ones(num_heads * head_dim), requires_grad=False)
-        self.k_norm = nn.Parameter(torch.ones(num_kv_heads * head_dim), requires_grad=False)
-        self.register_buffer("qk_freq", qk_freq.to(dtype=torch.float32, device=self.q_norm.device), persistent=False)
+        self.norm_per_head, self.chunk = norm_per_head, chunk
+        self.q_norm = nn.Parameter(torch.ones(head_dim if norm_per_head else num_heads * head_dim), requires_grad=False)
+        self.k_norm = nn.Parameter(torch.ones(head_dim if norm_per_head else num_kv_heads * head_dim), requires_grad=False)
+        if sinks:
+            self.sinks = nn.Parameter(torch.zeros(num_heads, dtype=torch.float32), requires_grad=False)      # (an operand of the fp32 softmax)
+        else:
+            self.register_parameter("sinks", None)
+        self.register_buffer("qk_freq", None if qk_freq is None else qk_freq.to(dtype=torch.float32, device=self.q_norm.device), persistent=False)
         self.register_buffer("value_freq", None if value_freq is None else value_freq.to(dtype=torch.float32, device=self.q_norm.device),
                              persistent=False)
         self.cache_runs = cache_runs
@@ -103,9 +112,10 @@ class GatedValueRotaryAttention(nn.Module):
             raise RuntimeError("this attention reads its keys from the paged cache: bind caches and give every sequence a block table")
         q, gate = ops.attn_rotary_prep(proj, self.q_norm.data, self.k_norm.data, self.eps, positions, self.qk_freq, self.qk_mag,
                                        self.rot_dims, self.value_freq, kc, vc, ctx.slot_mapping, self.num_heads, self.num_kv_heads,
-                                       self.head_dim, self.value_dim, self.gated, self.interleaved, self.interleaved)
+                                       self.head_dim, self.value_dim, self.gated, self.interleaved, self.interleaved, self.norm_per_head)
         return ops.attn_paged_any(q, kc, vc, ctx.cu_seqlens_q, ctx.context_lens, ctx.block_tables, self.scale, self.num_heads,
-                                  self.num_kv_heads, self.head_dim, self.value_dim, gate, self.value_freq, self.interleaved)
+                                  self.num_kv_heads, self.head_dim, self.value_dim, gate, self.value_freq, self.interleaved, chunk=self.chunk,
+                                  sinks=None if self.sinks is None else self.sinks.data)
 
 
 class WindowedBiasAttention(nn.Module):

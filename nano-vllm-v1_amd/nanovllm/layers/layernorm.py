@@ -6,6 +6,8 @@ it by nvh_residual_dyt (csrc/stream_f32.hip) over an fp32 residual stream.
 PostSumRMSNorm: an RMS norm taken AFTER the residual sum (the stream itself is the normed value), with the old stream's
 weight in the sum, a per-column scale of the sublayer's result and a weight stored around zero (nvh_residual_postnorm).
 
+SublayerOutputNorm: an RMS norm of a sublayer's RESULT, which then joins the stream with a multiplier (nvh_residual_subnorm).
+
 Interface of the reference's nanovllm/layers/layernorm.py:48-165: ``RMSNorm(hidden_size,
 eps)``, ``.weight``, ``forward(x)`` -> y, ``forward(x, residual)`` -> (y, new_residual).
 """
@@ -104,3 +106,22 @@ class PostSumRMSNorm(nn.Module):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         """The norm alone (no sum, the stream taken once): x fp32 [rows, dim] -> normed rows in the activation type (x is left as it is)."""
         return ops.residual_postnorm(x, self.weight.data, self.eps, None, None, None, 1.0, self.weight_offset, True, in_place=False)
+
+
+class SublayerOutputNorm(nn.Module):
+    """The close of a sublayer whose result, not its input, is normed:
+
+        x <- x + mult * weight * y / sqrt(mean(y^2) + eps),      y = the sublayer's result (a sum of up to three terms)
+
+    `weight` is ONE number for all columns (hidden_size None) or one per column.  The stream x is fp32 and is updated in place; `close`
+    returns it once more in the activation type, the input of a sublayer that reads the stream as it is."""
+
+    def __init__(self, eps: float, mult: float = 1.0, hidden_size: int | None = None) -> None:
+        super().__init__()
+        self.eps, self.mult = eps, float(mult)
+        self.weight = nn.Parameter(torch.ones(hidden_size or 1), requires_grad=False)
+        self.weight.weight_loader = lambda param, t: param.data.copy_(t.reshape(param.shape))
+
+    def close(self, x: torch.Tensor, a=None, a_scale: float = 1.0, b=None, b_scale: float = 1.0, c32=None, want_h: bool = True):
+        """a, b: terms of the result in the activation type (with their factors), c32: a term in fp32."""
+        return ops.residual_subnorm(x, self.weight.data, self.eps, self.mult, a, a_scale, b, b_scale, c32, want_h)

@@ -53,6 +53,60 @@ class GeneralizedDeltaRule(nn.Module):
         return ops.delta_post(o, self.norm.data, g, self.num_heads, self.head_dim, self.eps)
 
 
+class GatedDeltaRule(nn.Module):
+    """The gated delta rule ("Gated Delta Networks: Improving Mamba2 with Delta Rule", Yang, Kautz, Hatamizadeh): per head a matrix memory
+    S [key_dim, value_dim] in fp32 that decays as a whole and is corrected towards the token's value along its key,
+
+        S <- g S;      d = beta (v - S^T k);      S <- S + k d^T;      o = S^T q          (the read-out sees the token's own write)
+
+    with one decay g = exp(-exp(A_log) softplus(a + dt_bias)) and one write strength beta = sigmoid(b) per head and token.  q, k and v
+    first pass a short causal convolution over time per channel (`taps` wide, last tap on the current token, no bias, continued across
+    steps from the sequence's last taps - 1 inputs) and silu; q and k then become unit vectors per head, q also times key_dim^-1/2.
+    q / k heads may be fewer than value heads: value head h reads q / k head h // (num_heads // qk_heads).  The read-out of a head is
+    divided by its root mean square, multiplied by a weight row [value_dim] that the heads share, and by silu(gate).
+
+    forward takes column views of the fused projection output - qkv (the convolved channels q | k | v, adjoining), b, a [T, H], gate
+    [T, H * value_dim] - and returns [T, H * value_dim] in the activation type.  The scan is the generalized delta rule's
+    (csrc/delta_rule.hip): g on every key channel, the removal along k at rate beta g, the written key beta k."""
+
+    def __init__(self, num_heads: int, qk_heads: int, key_dim: int, value_dim: int, taps: int, eps: float, state_runs: int = 1):
+        super().__init__()
+        assert num_heads % qk_heads == 0 and taps >= 1
+        self.num_heads, self.qk_heads, self.key_dim, self.value_dim, self.taps, self.eps = num_heads, qk_heads, key_dim, value_dim, taps, eps
+        self.channel_sizes = [qk_heads * key_dim, qk_heads * key_dim, num_heads * value_dim]
+        self.conv_weight = nn.Parameter(torch.zeros(sum(self.channel_sizes), taps), requires_grad=False)
+        self.conv_weight.shard_ids = ["q", "k", "v"]
+        self.conv_weight.weight_loader = self._load_conv
+        self.dt_bias = nn.Parameter(torch.zeros(num_heads), requires_grad=False)
+        self.A_log = nn.Parameter(torch.zeros(num_heads), requires_grad=False)
+        self.norm = nn.Parameter(torch.ones(value_dim), requires_grad=False)
+        self.conv_inputs = _StatePool((max(taps - 1, 1), sum(self.channel_sizes)), state_runs)     # the last taps - 1 inputs of q | k | v per sequence
+        self.state_runs = state_runs
+        self.states: list = [None] * state_runs
+
+    def _load_conv(self, param: nn.Parameter, loaded_weight: torch.Tensor, shard_id):
+        i = self.conv_weight.shard_ids.index(shard_id)
+        dst = param.data.narrow(0, sum(self.channel_sizes[:i]), self.channel_sizes[i])
+        assert dst.shape == loaded_weight.shape, f"convolution of {shard_id!r}: {tuple(loaded_weight.shape)} does not fit {tuple(dst.shape)}"
+        dst.copy_(loaded_weight)
+
+    def state_shape(self) -> tuple[int, int, int]:
+        return self.num_heads, self.key_dim, self.value_dim
+
+    def projection_sizes(self) -> list[int]:
+        """Columns of the fused projection: q | k | v | b | a | gate."""
+        return self.channel_sizes + [self.num_heads, self.num_heads, self.num_heads * self.value_dim]
+
+    def forward(self, qkv, b, a, gate, run: int = 0) -> torch.Tensor:
+        ctx = get_context()
+        state = self.states[run]
+        if state is None or ctx.state_slots is None:
+            raise RuntimeError("the delta rule needs a bound state pool and a state slot per sequence")
+        o = ops.gated_delta_rule(qkv, b, a, self.conv_weight.data, self.dt_bias.data, self.A_log.data, self.conv_inputs.pool(run), state, ctx.state_slots,
+                                 ctx.cu_seqlens_q, ctx.context_lens, self.num_heads, self.qk_heads, self.key_dim, self.value_dim)
+        return ops.group_rmsnorm_gate(o, self.norm.data, self.value_dim, self.eps, gate, "silu", gate_first=False)
+
+
 class _StatePool(nn.Module):
     """A per-sequence fp32 state of fixed shape, one pool [slots, *shape] per pass (`states[run]`, bound by the runner)."""
 
@@ -244,3 +298,19 @@ class WKV(nn.Module):
         oq, ok, ow, ov = ops.wkv_prep(r, k, v, lowrank, self.w2.data, self.w0.data)
         o = self.memory(oq, ok, ow, ov, run, read_first=True, bonus=self.bonus.data)
         return ops.group_rmsnorm_gate(o, self.norm.data, self.head_dim, self.eps, gate, "silu", gate_first=False)
+
+
+class StreamConv(_StatePool):
+    """A short causal convolution of the fp32 residual stream over time, per column, added to the stream itself: what a sublayer reads
+    is h_t = x_t + sum_k w[:, k] x_(t - taps + 1 + k) (no bias; the last tap lies on the token itself; zeros before the sequence's
+    start).  The last taps - 1 rows of a sequence are carried from step to step in its state slot (fp32 [taps - 1, width])."""
+
+    def __init__(self, width: int, taps: int, state_runs: int = 1):
+        super().__init__((max(taps - 1, 1), width), state_runs)
+        self.width, self.taps = width, taps
+        self.weight = nn.Parameter(torch.zeros(width, taps), requires_grad=False)
+
+    def forward(self, x: torch.Tensor, run: int = 0) -> torch.Tensor:
+        """x fp32 [T, width] (left as it is) -> h in the activation type."""
+        ctx = get_context()
+        return ops.stream_conv(x, self.weight.data, self.pool(run), ctx.state_slots, ctx.cu_seqlens_q, ctx.context_lens)

@@ -71,3 +71,33 @@ def rotary_frequencies(dims: int, base: float, yarn: dict | None = None) -> tupl
         ramp = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
         out.append(f / factor * ramp + f * (1.0 - ramp))
     return torch.tensor(out, dtype=torch.float64).float(), 0.1 * math.log(factor) + 1.0
+
+
+def banded_frequencies(dims: int, base: float, scaling: dict | None = None) -> torch.Tensor:
+    """fp32 frequencies of the dims/2 rotation pairs, f_i = base^(-2i/dims), under a context-extension rule (float64 on the host):
+
+      scaling None                              the plain frequencies;
+      {factor}                                  position interpolation: every f_i / factor;
+      {factor, low, high, original}             the rule of Llama 3.1 by wavelength l = 2 pi / f: pairs with l < original / high keep
+                                                f, pairs with l > original / low take f / factor, and in between
+                                                s = (original / l - low) / (high - low) blends them, (1 - s) f / factor + s f."""
+    import math
+    freq = [base ** (-2.0 * i / dims) for i in range(dims // 2)]
+    if scaling:
+        factor = float(scaling["factor"])
+        if "original" in scaling:
+            low, high, original = float(scaling["low"]), float(scaling["high"]), float(scaling["original"])
+            out = []
+            for f in freq:
+                wavelength = 2.0 * math.pi / f
+                if wavelength < original / high:
+                    out.append(f)
+                elif wavelength > original / low:
+                    out.append(f / factor)
+                else:
+                    s = (original / wavelength - low) / (high - low)
+                    out.append((1.0 - s) * f / factor + s * f)
+            freq = out
+        else:
+            freq = [f / factor for f in freq]
+    return torch.tensor(freq, dtype=torch.float64).float()

@@ -22,6 +22,8 @@ _REGISTRY = {
     "DinatarForCausalLM": ("dinatar", "DinatarForCausalLM"),
     "Lakatar": ("lakatar", "LakatarForCausalLM"),
     "LakatarForCausalLM": ("lakatar", "LakatarForCausalLM"),
+    "Sokipel": ("sokipel", "SokipelForCausalLM"),
+    "SokipelForCausalLM": ("sokipel", "SokipelForCausalLM"),
 }
 
 

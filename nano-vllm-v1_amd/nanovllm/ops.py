@@ -658,29 +658,35 @@ def logit_softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
 
 def attn_rotary_prep(proj, q_norm, k_norm, eps: float, positions, qk_freq, qk_mag: float, rot_dims: int, v_freq, k_cache, v_cache,
                      slot_mapping, heads: int, kv_heads: int, dim: int, vdim: int, gated: bool = True, qk_interleaved: bool = False,
-                     v_interleaved: bool = False):
+                     v_interleaved: bool = False, norm_per_head: bool = False):
     """(q [T, H*dim], sigmoid gate fp32 [T, H] | None) from the fused projection rows [q | k | v | gate]; k and v go to their
-    cache rows (see nvh_attn_rotary_prep).  q_norm / k_norm None: no norm; rot_dims 0: no rotary."""
+    cache rows (see nvh_attn_rotary_prep).  q_norm / k_norm None: no norm; rot_dims 0: no rotary.  `norm_per_head`: the norm runs
+    over every head by itself, with weights [dim] that the heads share (else over the whole projection, weights of its size)."""
     f = _act_flag(proj, k_cache, v_cache) if q_norm is None else _act_flag(proj, q_norm, k_norm, k_cache, v_cache)
     t = proj.shape[0]
     assert proj.stride(1) == 1 and positions.dtype == torch.int64 and slot_mapping.dtype == torch.int32 and slot_mapping.numel() == t
     assert qk_freq is None or (qk_freq.dtype == F32 and qk_freq.numel() * 2 == rot_dims)
     assert v_freq is None or (v_freq.dtype == F32 and v_freq.numel() * 2 == vdim)
-    assert (q_norm is None and k_norm is None) or (q_norm.numel() == heads * dim and k_norm.numel() == kv_heads * dim)
+    assert (q_norm is None and k_norm is None) or (q_norm.numel() == k_norm.numel() == dim if norm_per_head else
+                                                    (q_norm.numel() == heads * dim and k_norm.numel() == kv_heads * dim))
     assert k_cache.is_contiguous() and v_cache.is_contiguous()
     q = torch.empty(t, heads * dim, dtype=proj.dtype, device=proj.device)
     gate = torch.empty(t, heads, dtype=F32, device=proj.device) if gated else None
     _hip.call("nvh_attn_rotary_prep", proj.data_ptr(), proj.stride(0), _p(q_norm), _p(k_norm), float(eps), positions.data_ptr(),
               _p(qk_freq), float(qk_mag), rot_dims, int(qk_interleaved), _p(v_freq), int(v_interleaved), q.data_ptr(), _p(gate),
-              k_cache.data_ptr(), v_cache.data_ptr(), slot_mapping.data_ptr(), k_cache.shape[1], t, heads, kv_heads, dim, vdim, f, _stream())
+              k_cache.data_ptr(), v_cache.data_ptr(), slot_mapping.data_ptr(), k_cache.shape[1], t, heads, kv_heads, dim, vdim,
+              int(norm_per_head and q_norm is not None), f, _stream())
     return q, gate
 
 
 def attn_paged_any(q, k_cache, v_cache, cu_seqlens_q, context_lens, block_tables, scale: float, heads: int, kv_heads: int, dim: int,
-                   vdim: int, gate=None, v_freq=None, v_interleaved: bool = False, slopes=None, window: int = 0, keep_first: int = 0) -> torch.Tensor:
+                   vdim: int, gate=None, v_freq=None, v_interleaved: bool = False, slopes=None, window: int = 0, keep_first: int = 0,
+                   chunk: int = 0, sinks=None) -> torch.Tensor:
     """Causal attention of the packed queries q [T, H*dim] over paged caches, keys [pages, page, G, dim] and values
     [pages, G, vdim, page] (transposed within a page, as attn_rotary_prep stores them); out [T, H*vdim].  `slopes` (fp32 [H]):
-    score -= slope * distance; `window` > 0: a query sees the last `window` positions and the first `keep_first`."""
+    score -= slope * distance; `window` > 0: a query sees the last `window` positions and the first `keep_first`; `chunk` > 0: a
+    query sees only the keys of its own block of `chunk` positions (counted from the sequence's start); `sinks` (fp32 [H]): a logit
+    per head that joins the softmax's denominator once, with no key and no value."""
     f = _act_flag(q, k_cache, v_cache)
     t = q.shape[0]
     batch = context_lens.numel()
@@ -691,13 +697,15 @@ def attn_paged_any(q, k_cache, v_cache, cu_seqlens_q, context_lens, block_tables
     assert cu_seqlens_q is not None or t == batch
     assert gate is None or (gate.dtype == F32 and gate.shape == (t, heads) and gate.is_contiguous())
     assert slopes is None or (slopes.dtype == F32 and slopes.numel() == heads and slopes.is_contiguous() and slopes.is_cuda)
+    assert sinks is None or (sinks.dtype == F32 and sinks.numel() == heads and sinks.is_contiguous() and sinks.is_cuda)
     out = torch.empty(t, heads * vdim, dtype=q.dtype, device=q.device)
     # one-query steps that would leave most of the chip idle spread a sequence's key tiles over several workgroups: scratch for their rows
     ws_bytes = int(_hip.lib().nvh_attn_paged_any_parts_bytes(batch, t, heads, kv_heads, dim, vdim, k_cache.shape[1], int(v_freq is not None), f))
     ws = torch.empty(ws_bytes // 4, dtype=F32, device=q.device) if ws_bytes else None
     _hip.call("nvh_attn_paged_any", q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _p(cu_seqlens_q), context_lens.data_ptr(),
               block_tables.data_ptr(), block_tables.stride(0), batch, t, k_cache.shape[1], heads, kv_heads, dim, vdim, float(scale),
-              _p(gate), _p(v_freq), int(v_interleaved), _p(slopes), int(window), int(keep_first), out.data_ptr(), _p(ws), ws_bytes, f, _stream())
+              _p(gate), _p(v_freq), int(v_interleaved), _p(slopes), int(window), int(keep_first), int(chunk), _p(sinks), out.data_ptr(), _p(ws), ws_bytes,
+              f, _stream())
     return out
 
 
@@ -720,7 +728,35 @@ def delta_rule(r, k, v, a_raw, lowrank, w2, w0, a_bias, state, slots, cu_seqlens
               t, heads, dk, rank, float(decay_scale), f, _stream())
     out = torch.empty(t, heads * dk, dtype=F32, device=r.device)
     _hip.call("nvh_delta_scan", pack.data_ptr(), state.data_ptr(), slots.data_ptr(), _p(cu_seqlens_q), context_lens.data_ptr(),
-              out.data_ptr(), batch, heads, dk, _stream())
+              out.data_ptr(), batch, heads, dk, dk, _stream())
+    return out
+
+
+def gated_delta_rule(qkv, b, a, conv_w, dt_bias, a_log, conv_state, state, slots, cu_seqlens_q, context_lens, heads: int, qk_heads: int,
+                     dk: int, dv: int) -> torch.Tensor:
+    """One step of the gated delta rule over the packed tokens: fp32 outputs [T, H*dv].  `qkv`: the column view q | k | v of the
+    projection rows (qk_heads*dk, qk_heads*dk, heads*dv channels), convolved over time with `conv_w` [C, taps] (continued from
+    `conv_state` [slots, taps - 1, C] fp32, then brought up to date) and passed through silu; `b`, `a`: column views [T, H] of the
+    write-strength and decay logits.  `state` [slots, H, dk, dv] fp32 is read (unless the sequence starts in this step) and left
+    updated."""
+    f = _act_flag(qkv, b, a, conv_w, dt_bias, a_log)
+    t, c = qkv.shape[0], 2 * qk_heads * dk + heads * dv
+    taps = conv_w.shape[1]
+    batch = context_lens.numel()
+    assert qkv.shape[1] == c and qkv.stride(1) == 1 and b.shape == (t, heads) and a.shape == (t, heads) and b.stride(1) == 1 and a.stride(1) == 1
+    assert conv_w.shape == (c, taps) and conv_w.is_contiguous() and dt_bias.numel() == heads and a_log.numel() == heads and heads % qk_heads == 0
+    assert taps == 1 or (conv_state.dtype == F32 and conv_state.is_contiguous() and tuple(conv_state.shape[1:]) == (taps - 1, c))
+    assert state.dtype == F32 and state.is_contiguous() and tuple(state.shape[1:]) == (heads, dk, dv) and slots.dtype == torch.int32
+    assert context_lens.dtype == torch.int32 and (cu_seqlens_q is None or cu_seqlens_q.dtype == torch.int32)
+    pack = torch.empty(t, heads, 5 * dk + dv, dtype=F32, device=qkv.device)
+    _hip.call("nvh_gated_delta_prep", qkv.data_ptr(), qkv.stride(0), b.data_ptr(), b.stride(0), a.data_ptr(), a.stride(0), conv_w.data_ptr(),
+              dt_bias.data_ptr(), a_log.data_ptr(), _p(conv_state), slots.data_ptr(), _p(cu_seqlens_q), context_lens.data_ptr(), pack.data_ptr(),
+              batch, t, taps, heads, qk_heads, dk, dv, f, _stream())
+    _hip.call("nvh_conv_state_update", qkv.data_ptr(), qkv.stride(0), _p(conv_state), slots.data_ptr(), _p(cu_seqlens_q), context_lens.data_ptr(), batch,
+              taps, c, f, _stream())
+    out = torch.empty(t, heads * dv, dtype=F32, device=qkv.device)
+    _hip.call("nvh_delta_scan", pack.data_ptr(), state.data_ptr(), slots.data_ptr(), _p(cu_seqlens_q), context_lens.data_ptr(),
+              out.data_ptr(), batch, heads, dk, dv, _stream())
     return out
 
 
@@ -787,6 +823,44 @@ def residual_postnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, y=None,
     h = torch.empty(rows, dim, dtype=weight.dtype, device=x.device) if want_h else None
     _hip.call("nvh_residual_postnorm", _p(y), y.stride(0) if y is not None else 0, _p(y32), y32.stride(0) if y32 is not None else 0, _p(layer_scale),
               float(alpha), x.data_ptr(), int(in_place), weight.data_ptr(), float(weight_offset), float(eps), _p(h), dim, rows, dim, f, _stream())
+    return h
+
+
+def residual_subnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, mult: float = 1.0, a=None, a_scale: float = 1.0, b=None, b_scale: float = 1.0,
+                     c32=None, want_h: bool = True):
+    """x <- x + mult * weight * y / sqrt(mean(y^2) + eps) in place (fp32 rows), y = a_scale a + b_scale b + c32: a sublayer's result is
+    normed before it joins the stream.  a, b: rows of the activation type, c32: fp32 rows (any may be absent); weight: one number or
+    one per column.  Returns the new x in the activation type (the next sublayer's input), or None."""
+    assert x.dtype == F32 and x.is_contiguous() and x.dim() == 2 and (a is not None or b is not None or c32 is not None)
+    rows, dim = x.shape
+    typed = [t for t in (a, b, weight) if t is not None]
+    f = _act_flag(*typed)
+    for t in (a, b, c32):
+        assert t is None or (t.shape == (rows, dim) and t.stride(1) == 1)
+    assert c32 is None or (c32.dtype == F32 and c32.is_cuda)
+    assert weight.numel() in (1, dim) and weight.is_contiguous()
+    h = torch.empty(rows, dim, dtype=weight.dtype, device=x.device) if want_h else None
+    _hip.call("nvh_residual_subnorm", _p(a), a.stride(0) if a is not None else 0, float(a_scale), _p(b), b.stride(0) if b is not None else 0, float(b_scale),
+              _p(c32), c32.stride(0) if c32 is not None else 0, float(mult), weight.data_ptr(), weight.numel(), float(eps), x.data_ptr(), _p(h), dim, rows, dim,
+              f, _stream())
+    return h
+
+
+def stream_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor | None, slots, cu_seqlens_q, context_lens) -> torch.Tensor:
+    """h_t = x_t + sum_k weight[:, k] x_(t - taps + 1 + k) over the fp32 stream x [T, dim] (the last tap on the token itself), in weight's
+    type.  Rows before this step come from `state` [slots, taps - 1, dim] fp32 (zeros at a sequence's start), which is then brought up
+    to date with this step's rows."""
+    f = _act_flag(weight)
+    t, dim = x.shape
+    taps = weight.shape[1]
+    batch = context_lens.numel()
+    assert x.dtype == F32 and x.is_contiguous() and weight.shape == (dim, taps) and weight.is_contiguous()
+    assert taps == 1 or (state.dtype == F32 and state.is_contiguous() and tuple(state.shape[1:]) == (taps - 1, dim))
+    assert slots.dtype == torch.int32 and context_lens.dtype == torch.int32 and (cu_seqlens_q is None or cu_seqlens_q.dtype == torch.int32)
+    h = torch.empty(t, dim, dtype=weight.dtype, device=x.device)
+    _hip.call("nvh_stream_conv", x.data_ptr(), weight.data_ptr(), _p(state), slots.data_ptr(), _p(cu_seqlens_q), context_lens.data_ptr(), h.data_ptr(), dim,
+              batch, t, taps, dim, f, _stream())
+    _hip.call("nvh_conv_state_update", x.data_ptr(), dim, _p(state), slots.data_ptr(), _p(cu_seqlens_q), context_lens.data_ptr(), batch, taps, dim, 1, _stream())
     return h
 
 
@@ -981,8 +1055,9 @@ def moe_route(logits: torch.Tensor, top: int):
     return ids, weights
 
 
-def moe_route_linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, top: int, want_logits: bool = False):
-    """moe_route of the fp32 logits x @ weight^T + bias, formed inside the same launch: (ids, weights[, logits])."""
+def moe_route_linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, top: int, want_logits: bool = False, sigmoid_scores: bool = False):
+    """moe_route of the fp32 logits x @ weight^T + bias, formed inside the same launch: (ids, weights[, logits]).  `sigmoid_scores`: the
+    weights are the picked experts' own sigmoid(logit), not renormalised."""
     f = _act_flag(x, weight) if bias is None else _act_flag(x, weight, bias)
     t, k = x.shape
     e = weight.shape[0]
@@ -990,7 +1065,8 @@ def moe_route_linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor |
     ids = torch.empty(t, top, dtype=torch.int32, device=x.device)
     weights = torch.empty(t, top, dtype=F32, device=x.device)
     logits = torch.empty(t, e, dtype=F32, device=x.device) if want_logits else None
-    _hip.call("nvh_moe_route_linear", x.data_ptr(), x.stride(0), weight.data_ptr(), _p(bias), ids.data_ptr(), weights.data_ptr(), _p(logits), t, e, k, top, f, _stream())
+    _hip.call("nvh_moe_route_linear", x.data_ptr(), x.stride(0), weight.data_ptr(), _p(bias), ids.data_ptr(), weights.data_ptr(), _p(logits), t, e, k, top,
+              int(sigmoid_scores), f, _stream())
     return (ids, weights, logits) if want_logits else (ids, weights)
 
 
@@ -1019,17 +1095,31 @@ def linear_grouped(x: torch.Tensor, weight: torch.Tensor, plan: dict, gather: bo
     return y
 
 
-def moe_combine(y: torch.Tensor, plan: dict, weights: torch.Tensor, shared: torch.Tensor | None = None, shared_gate: torch.Tensor | None = None) -> torch.Tensor:
+def glu_clamp_pairs(gate_up: torch.Tensor, plan: dict, weights: torch.Tensor | None, limit: float, alpha: float = 1.702) -> torch.Tensor:
+    """The experts' activation over the rows [G | U] of the first grouped product where a pair's routing weight w (fp32 [T, top]; None:
+    1) multiplies the expert's input: g = min(w G, limit), u = clamp(w U, -limit, limit), y = g sigmoid(alpha g) (u + 1)."""
+    f = _act_flag(gate_up)
+    pairs, inter = gate_up.shape[0], gate_up.shape[1] // 2
+    assert gate_up.dim() == 2 and gate_up.stride(1) == 1 and pairs == plan["pairs"] and (weights is None or (weights.dtype == F32 and weights.is_contiguous() and weights.numel() == pairs))
+    y = torch.empty(pairs, inter, dtype=gate_up.dtype, device=gate_up.device)
+    _hip.call("nvh_glu_clamp_pairs", gate_up.data_ptr(), gate_up.stride(0), plan["pos_of_pair"].data_ptr(), _p(weights), y.data_ptr(), inter, pairs, inter,
+              float(limit), float(alpha), f, _stream())
+    return y
+
+
+def moe_combine(y: torch.Tensor, plan: dict, weights: torch.Tensor | None, shared: torch.Tensor | None = None, shared_gate: torch.Tensor | None = None,
+                top: int | None = None) -> torch.Tensor:
     """fp32 [T, dim]: every token's weighted sum of its choices' rows of y (in choice order), plus `shared` [T, dim], which is
-    multiplied by sigmoid(shared_gate[t]) when a gate logit per token (fp32 [T] or a column view) is given."""
+    multiplied by sigmoid(shared_gate[t]) when a gate logit per token (fp32 [T] or a column view) is given.  weights None (then
+    `top` says how many choices a token has): a plain sum."""
     f = _act_flag(y) if shared is None else _act_flag(y, shared)
-    t, top = weights.shape
+    t, top = weights.shape if weights is not None else (plan["pairs"] // top, top)
     dim = y.shape[1]
-    assert y.stride(1) == 1 and weights.dtype == F32 and weights.is_contiguous() and y.shape[0] == t * top
+    assert y.stride(1) == 1 and (weights is None or (weights.dtype == F32 and weights.is_contiguous())) and y.shape[0] == t * top
     assert shared is None or (shared.shape == (t, dim) and shared.stride(1) == 1)
     assert shared_gate is None or (shared is not None and shared_gate.dtype == F32 and shared_gate.numel() == t and shared_gate.is_cuda)
     out = torch.empty(t, dim, dtype=F32, device=y.device)
-    _hip.call("nvh_moe_combine", y.data_ptr(), y.stride(0), plan["pos_of_pair"].data_ptr(), weights.data_ptr(), _p(shared),
+    _hip.call("nvh_moe_combine", y.data_ptr(), y.stride(0), plan["pos_of_pair"].data_ptr(), _p(weights), _p(shared),
               shared.stride(0) if shared is not None else 0, _p(shared_gate), shared_gate.reshape(t, -1).stride(0) if shared_gate is not None else 0,
               out.data_ptr(), t, dim, top, f, _stream())
     return out
