@@ -49,7 +49,7 @@ def config(layers, width=96, vocab=131, taps=3, scale=4.0, mult=0.6, cap=20.0, e
 
 
 CFG_MIX = config([DEL_A, PAR_A, ATT_A, PAR_B, DEL_B])
-CFG_FLAT = config([ATT_B, DEL_B, PAR_A, DEL_C], width=128, vocab=200, taps=5, scale=2.0, mult=1.2, cap=35.0, eps=1e-6)
+CFG_FLAT = config([ATT_B, DEL_B, PAR_A, DEL_C], width=128, vocab=200, taps=5, scale=2.0, mult=0.5, cap=35.0, eps=1e-6)
 
 
 def random_weights(cfg: dict, seed: int, calm: bool = False) -> dict:
@@ -99,7 +99,7 @@ def random_weights(cfg: dict, seed: int, calm: bool = False) -> dict:
 
     mat("embed", V, D, 1.0)
     if calm:
-        W["embed"][:, 0] = 3.0
+        W["embed"][:, 0] = 24.0 / cfg["embedding"]["scale"]            # (large beside what the layers add to it on the way)
     mat("head", V, D)
     one("final.norm")
     for i, L in enumerate(cfg["layers"]):
@@ -125,7 +125,7 @@ def random_weights(cfg: dict, seed: int, calm: bool = False) -> dict:
             mat(f"{p}mlp.e{e}.down", D, ff)
         if calm:
             mat(p + "mlp.router", E, D, 0.02 / math.sqrt(D))
-            W[p + "mlp.router"][:, 0] = torch.linspace(-0.4, 0.4, E)[torch.randperm(E, generator=g)]
+            W[p + "mlp.router"][:, 0] = torch.linspace(-0.15, 0.15, E)[torch.randperm(E, generator=g)]
         else:
             mat(p + "mlp.router", E, D, 0.5 / math.sqrt(D))
     return {k: v.to(torch.bfloat16) for k, v in W.items()}
@@ -573,7 +573,7 @@ def test_a_far_key_decides_wherever_it_lies(tmp_path, dtype, beside):
     W = dict(case.W)
     sink = "l0.mix.left.sink" if beside else "l0.mix.sink"
     W[sink] = torch.full_like(W[sink], -30.0)
-    assert rel_err(R.forward(W, cfg, base[:n - 1] + [899]).numpy()[-1:], plain) > 0.1           # without the sink the logits are others
+    assert rel_err(R.forward(W, cfg, base[:n - 1] + [899]).numpy()[-1:], plain) > 0.05          # without the sink the logits are others
     rp = case.replay(dtype, max_tokens=1300)
     try:
         for far in (0, 3, 255, 256, 257, 399, 400, 401, 511, 512, n - 2):
@@ -603,7 +603,7 @@ def test_the_memory_carries_a_token_from_far_back(tmp_path):
     w["l0.mix.A_log"] = torch.full_like(w["l0.mix.A_log"], -7.0)
     w["l0.canon1"][0] = 0
     w["l0.mix.b"] = w["l0.mix.b"] * 0.1
-    w["l0.mix.b"][:, 0] = -0.4                                          # weak writes: a write also wears off what lies along its key
+    w["l0.mix.b"][:, 0] = -0.2                                          # weak writes: a write also wears off what lies along its key
     case = Case(tmp_path, cfg, weights=w)
     toks = tokens_of(cfg, 400, 8)
     changed = [(toks[0] + 1) % 90] + toks[1:]
