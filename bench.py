@@ -520,11 +520,30 @@ def _lakatar_cfg(z):
     return {"architecture": "Lakatar", "vocab": z["vocab"], "width": w, "norm": {"eps": 1e-6}, "postln_alpha": 2.0, "layers": layers}
 
 
+def _sokipel_cfg(z):
+    """Gated-delta-rule, parallel (sink attention beside a gated delta rule) and chunked sink-attention layers in turn, a four-tap
+    convolution of the stream in front of every mixer, every feed-forward a mixture of 16 capped experts of which a token takes 4
+    (together as wide as the dense feed-forward of the size)."""
+    w, hd = z["width"], z["head_dim"]
+    bands = {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}
+    delta = {"heads": w // 128, "kv_heads": max(w // 256, 1), "dim": 128, "vdim": 128, "conv": 4}
+    left = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": hd, "vdim": hd, "scale": hd ** -0.5, "rot": {"base": 1e6, "dims": hd // 2, "scaling": {"factor": 4.0}}}
+    right = {"heads": max(w // 256, 1), "kv_heads": max(w // 512, 1), "dim": 128, "vdim": 128, "conv": 4}
+    chunked = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": hd, "vdim": hd, "scale": hd ** -0.5, "rot": {"base": 1e6, "dims": hd, "scaling": bands},
+               "mask": {"size": 512}}
+    mixers = [("delta", delta), ("parallel", {"left": left, "left_scale": 0.6, "right": right, "right_scale": 0.9}), ("attention", chunked)]
+    moe = {"kind": "moe", "expert": {"ff": z["ff"] // 4, "limit": 7.0}, "router": {"experts": 16, "top": 4}}
+    return {"architecture": "Sokipel", "vocab": z["vocab"], "width": w, "norm": {"eps": 1e-6}, "embedding": {"scale": 1.0}, "residual_mult": 0.5,
+            "logit_softcap": 30.0, "canon": {"taps": 4},
+            "layers": [{"type": mixers[i % 3][0], "mixer": mixers[i % 3][1], "mlp": moe} for i in range(z["layers"])]}
+
+
 HYBRID_DESIGNS = {
     # --hybrid-design: (the design, the closest model the engine already serves)
     "lamutar": (("lamutar", _lamutar_cfg), ("qwen3", _qwen3_cfg)),
     "dinatar": (("dinatar", _dinatar_cfg), ("lamutar", _lamutar_cfg)),
     "lakatar": (("lakatar", _lakatar_cfg), ("dinatar", _dinatar_cfg)),
+    "sokipel": (("sokipel", _sokipel_cfg), ("dinatar", _dinatar_cfg)),
 }
 
 
@@ -533,7 +552,9 @@ def hybrid_compare(args):
     stream + captured decode graphs) beside the closest model the engine serves at equal width, heads, feed-forward size, depth and
     vocabulary: Lamutar (delta-rule and attention layers in turn) beside Qwen3 (native executor), or Dinatar (windowed attention +
     Mamba-2, HGRN2, gated linear attention; dense and expert feed-forwards) beside Lamutar, or Lakatar (RWKV-style time mix, latent
-    attention, retention; score-routed experts; norms after the sums) beside Dinatar.  Random weights, bf16.  One JSON line."""
+    attention, retention; score-routed experts; norms after the sums) beside Dinatar, or Sokipel (gated delta rule, sink attention in
+    chunks and beside a delta rule, a convolution of the stream, capped experts fed with their weight) beside Dinatar.  Random weights,
+    bf16.  One JSON line."""
     import tempfile
     from nanovllm.config import Config
     from nanovllm.engine.model_runner import ModelRunner
@@ -578,7 +599,7 @@ def main():
     ap.add_argument("--hybrid-compare", action="store_true",
                     help="instead of the headline workload: a hybrid design beside the closest model at equal layer sizes (see hybrid_compare)")
     ap.add_argument("--hybrid-design", default="lamutar", choices=sorted(HYBRID_DESIGNS),
-                    help="lamutar (beside Qwen3; the default), dinatar (beside Lamutar) or lakatar (beside Dinatar)")
+                    help="lamutar (beside Qwen3; the default), dinatar (beside Lamutar), lakatar (beside Dinatar) or sokipel (beside Dinatar)")
     ap.add_argument("--hybrid-sizes", default="", help="comma-separated subset of " + ",".join(HYBRID_SIZES))
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)

@@ -56,33 +56,33 @@ struct GatedDeltaPrepArgs {
 
 __device__ __forceinline__ float softplusf_(float x) { return x > 20.f ? x : log1pf(expf(x)); }
 
-// One workgroup per token.  The convolved, activated channels meet in LDS; a wave per q / k head sums its squares; then every
-// head's row is written.
+// One workgroup per (token, value head): the convolved, activated channels of the head's q / k group and of its own v meet in LDS,
+// two waves sum the squares of q and k, then the head's row is written.  (Heads that share a q / k group convolve it again each: a
+// few hundred channels, against a launch that would otherwise have as many workgroups as tokens only.)
 template <typename A>
 __global__ __launch_bounds__(256) void gated_delta_prep_kernel(GatedDeltaPrepArgs p) {
-    extern __shared__ float sh[];                            // [C] channels, then [2 G] inverse lengths, then [H] beta, [H] g
+    extern __shared__ float sh[];                            // [dk] q, [dk] k, [dv] v of this head, then the two inverse lengths
     const int64_t t = blockIdx.x;
-    const int nqk = p.G * p.dk, C = 2 * nqk + p.H * p.dv, taps = p.taps;
-    float* inv = sh + C;
-    float* beta = inv + 2 * p.G;
-    float* dec = beta + p.H;
-    int seq = 0;
+    const int h = blockIdx.y, dk = p.dk, dv = p.dv, g = h / (p.H / p.G);
+    const int nqk = p.G * dk, C = 2 * nqk + p.H * dv, taps = p.taps, n = 2 * dk + dv;
+    float* inv = sh + n;
+    int seq = (int)t;
     if (p.cu_seqlens_q) {
         int lo_b = 0, hi_b = p.batch;                        // the sequence whose rows hold token t
         while (hi_b - lo_b > 1) {
             const int mid = (lo_b + hi_b) >> 1;
-            if (p.cu_seqlens_q[mid] <= t) lo_b = mid; else hi_b = mid;
+            if (p.cu_seqlens_q[mid] <= t) lo_b = mid;
+            else hi_b = mid;
         }
         seq = lo_b;
-    } else {
-        seq = (int)t;
     }
     const int lo = p.cu_seqlens_q ? p.cu_seqlens_q[seq] : seq, hi = p.cu_seqlens_q ? p.cu_seqlens_q[seq + 1] : seq + 1;
     const int j = (int)t - lo;
     const int slot = p.slots[seq];
     const bool carried = slot >= 0 && p.context_lens[seq] != hi - lo;
     const float* st = carried ? p.conv_state + (int64_t)slot * (taps - 1) * C : nullptr;
-    for (int c = threadIdx.x; c < C; c += 256) {
+    for (int e = threadIdx.x; e < n; e += 256) {
+        const int c = e < dk ? g * dk + e : (e < 2 * dk ? nqk + g * dk + (e - dk) : 2 * nqk + h * dv + (e - 2 * dk));      // the channel of the row
         float acc = 0.f;
         for (int k = 0; k < taps; ++k) {                     // tap k multiplies the input taps - 1 - k tokens back
             const int back = taps - 1 - k, src = j - back;
@@ -91,41 +91,31 @@ __global__ __launch_bounds__(256) void gated_delta_prep_kernel(GatedDeltaPrepArg
             else if (st) in = st[(int64_t)(taps - 1 + src) * C + c];
             acc = __builtin_fmaf(ldf((const A*)p.conv_w, (int64_t)c * taps + k), in, acc);
         }
-        sh[c] = acc / (1.0f + expf(-acc));
+        sh[e] = acc / (1.0f + expf(-acc));
     }
-    for (int h = threadIdx.x; h < p.H; h += 256) {
-        beta[h] = sigmoidf_(ldf((const A*)p.b, t * p.b_stride + h));
-        const float dt = softplusf_(ldf((const A*)p.a, t * p.a_stride + h) + ldf((const A*)p.dt_bias, h));
-        dec[h] = expf(-expf(ldf((const A*)p.a_log, h)) * dt);
-    }
+    const float beta = sigmoidf_(ldf((const A*)p.b, t * p.b_stride + h));
+    const float dec = expf(-expf(ldf((const A*)p.a_log, h)) * softplusf_(ldf((const A*)p.a, t * p.a_stride + h) + ldf((const A*)p.dt_bias, h)));
     __syncthreads();
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    for (int g = wave; g < 2 * p.G; g += 4) {                // q heads, then k heads (they lie one after the other)
+    if (wave < 2) {                                          // q, k
         float ss = 0.f;
-        for (int i = lane; i < p.dk; i += 64) ss += sh[g * p.dk + i] * sh[g * p.dk + i];
+        for (int i = lane; i < dk; i += 64) ss += sh[wave * dk + i] * sh[wave * dk + i];
         ss = wave_sum(ss);
-        if (lane == 0) inv[g] = 1.0f / sqrtf(ss + 1e-6f);
+        if (lane == 0) inv[wave] = 1.0f / sqrtf(ss + 1e-6f);
     }
     __syncthreads();
-    const int dk = p.dk, dv = p.dv, row = 5 * dk + dv, per = p.H / p.G;
-    const float qs = 1.0f / sqrtf((float)dk);
-    float* out = p.out + t * (int64_t)p.H * row;
-    for (int e = threadIdx.x; e < p.H * row; e += 256) {
-        const int h = e / row, r = e - h * row, g = h / per;
-        float v;
-        if (r >= 5 * dk) {
-            v = sh[2 * nqk + h * dv + (r - 5 * dk)];
-        } else {
-            const int part = r / dk, i = r - part * dk;
-            const float ku = sh[nqk + g * dk + i] * inv[p.G + g];
-            if (part == 0) v = sh[g * dk + i] * inv[g] * qs;
-            else if (part == 1) v = beta[h] * ku;
-            else if (part == 2) v = dec[h];
-            else if (part == 3) v = ku;
-            else v = beta[h] * dec[h] * ku;
-        }
-        out[e] = v;
+    const int row = 5 * dk + dv;
+    const float qs = inv[0] / sqrtf((float)dk), ks = inv[1];
+    float* out = p.out + (t * p.H + h) * (int64_t)row;
+    for (int i = threadIdx.x; i < dk; i += 256) {
+        const float ku = sh[dk + i] * ks;
+        out[i] = sh[i] * qs;
+        out[dk + i] = beta * ku;
+        out[2 * dk + i] = dec;
+        out[3 * dk + i] = ku;
+        out[4 * dk + i] = beta * dec * ku;
     }
+    for (int i = threadIdx.x; i < dv; i += 256) out[5 * dk + i] = sh[2 * dk + i];
 }
 
 template <typename A>
@@ -398,14 +388,15 @@ extern "C" int32_t nvh_gated_delta_prep(const void* qkv, int64_t qkv_stride, con
     NVH_REQUIRE(cu_seqlens_q || num_tokens == batch, NVH_EINVAL, "nvh_gated_delta_prep: one token per sequence without cu_seqlens_q");
     const int64_t channels = 2 * qk_heads * dk + heads * dv;
     NVH_REQUIRE(qkv_stride >= channels, NVH_EINVAL, "nvh_gated_delta_prep: projection row too short");
-    const size_t lds = sizeof(float) * (size_t)(channels + 2 * qk_heads + 2 * heads);
-    NVH_REQUIRE(lds <= 64 * 1024, NVH_ENOSYS, "nvh_gated_delta_prep: %ld channels above the kernel's limit", (long)channels);
+    const size_t lds = sizeof(float) * (size_t)(2 * dk + dv + 2);
+    NVH_REQUIRE(lds <= 64 * 1024 && heads <= 65535, NVH_ENOSYS, "nvh_gated_delta_prep: head sizes %ld + %ld above the kernel's limit", (long)dk, (long)dv);
     if (num_tokens == 0 || batch == 0) return NVH_OK;
     GatedDeltaPrepArgs p{qkv, qkv_stride, b, a, b_stride, a_stride, conv_w, dt_bias, a_log, conv_state, slots, cu_seqlens_q, context_lens, out,
                          (int)batch, (int)taps, (int)heads, (int)qk_heads, (int)dk, (int)dv};
     hipStream_t st = (hipStream_t)stream;
-    if (act_f32) gated_delta_prep_kernel<float><<<dim3((unsigned)num_tokens), 256, lds, st>>>(p);
-    else gated_delta_prep_kernel<bf16><<<dim3((unsigned)num_tokens), 256, lds, st>>>(p);
+    const dim3 grid((unsigned)num_tokens, (unsigned)heads);
+    if (act_f32) gated_delta_prep_kernel<float><<<grid, 256, lds, st>>>(p);
+    else gated_delta_prep_kernel<bf16><<<grid, 256, lds, st>>>(p);
     NVH_CHECK_LAUNCH("nvh_gated_delta_prep");
     return NVH_OK;
 }

@@ -755,3 +755,19 @@ def test_the_replay_program_steps_through_a_schedule(tmp_path, mix_case_calm):
         for n, w in want.items():
             got = np.fromfile(out / f"{n}.f32", dtype="<f4").reshape(-1, CFG_MIX["vocab"])
             assert got.shape == w.shape and rel_err(got, w) < TOL[dtype], (dtype, n)
+
+
+def test_the_sample_config_is_served_with_random_weights():
+    """model_configs/sokipel-mixed-1k (layer sizes of a real model; no checkpoint, so the engine draws weights): prompts of unequal
+    length are prefilled in chunks and decoded from captured graphs."""
+    from conftest import ROOT
+    from nanovllm import LLM, SamplingParams
+    llm = LLM(str(ROOT / "nano-vllm-v1_amd" / "model_configs" / "sokipel-mixed-1k"), max_num_seqs=4, max_num_batched_tokens=256, max_model_len=1024,
+              num_kvcache_blocks=12, chunked_prefill=True)
+    try:
+        prompts = [torch.randint(0, 32768, (n,), generator=torch.Generator().manual_seed(n)).tolist() for n in (600, 3, 130)]
+        outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True), use_tqdm=False)
+        again = llm.generate(prompts[1:2], SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True), use_tqdm=False)
+    finally:
+        llm.exit()
+    assert all(len(o["token_ids"]) == 8 for o in outs) and again[0]["token_ids"] == outs[1]["token_ids"]
