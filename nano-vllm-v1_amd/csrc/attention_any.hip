@@ -15,7 +15,7 @@
 //                         j < keep_first; key tiles that no query of a workgroup can see are never loaded.
 //                         Optional: chunks, query i sees key j <= i only when both lie in the same block of `chunk`
 //                         positions counted from the sequence's start; and a sink per head, a learned logit that joins the
-//                         softmax's denominator once, unscaled, with no key and no value (it is the state a row starts from:
+//                         softmax's denominator as one more term, as it is, standing for no token (it is the state a row starts from:
 //                         maximum = sink, sum = 1, output = 0).
 //                         Steps in which every sequence brings one query: the heads that share a KV head share a workgroup
 //                         (groups of more than 16 heads in parts); when that leaves most of the chip idle, a sequence's key

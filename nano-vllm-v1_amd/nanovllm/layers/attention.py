@@ -74,8 +74,8 @@ class GatedValueRotaryAttention(nn.Module):
     q and k projections (or, with `norm_per_head`, over every head by itself with a weight row [dim] that the heads share) run
     with the rotary in one launch (nvh_attn_rotary_prep), attention in a second (nvh_attn_paged_any).  `chunk` > 0: a query
     sees only the earlier tokens of its own block of `chunk` positions, blocks counted from the sequence's start.  `sinks`: a
-    learned logit per head (parameter `sinks`, fp32) joins the softmax's denominator once - it has no key and no value and is
-    not multiplied by `scale` - so a head can give weight to nothing.  A module that serves several passes of a looped stack
+    learned logit per head (parameter `sinks`, fp32) is one more term exp(sink) of the softmax's denominator - it stands for no
+    token, carries no value and is taken as it is, without `scale` - so a head can give weight to nothing.  A module that serves several passes of a looped stack
     owns one cache per pass:
     `k_caches[run]` [pages, page, G, dim] and `v_caches[run]` [pages, G, vdim, page] (values lie transposed within a page),
     bound by the runner (`cache_runs` of each)."""

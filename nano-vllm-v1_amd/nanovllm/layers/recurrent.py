@@ -57,7 +57,7 @@ class GatedDeltaRule(nn.Module):
     """The gated delta rule ("Gated Delta Networks: Improving Mamba2 with Delta Rule", Yang, Kautz, Hatamizadeh): per head a matrix memory
     S [key_dim, value_dim] in fp32 that decays as a whole and is corrected towards the token's value along its key,
 
-        S <- g S;      d = beta (v - S^T k);      S <- S + k d^T;      o = S^T q          (the read-out sees the token's own write)
+        S <- g S;      d = beta (v - S^T k);      S <- S + k d^T;      o = S^T q          (o is taken after the update)
 
     with one decay g = exp(-exp(A_log) softplus(a + dt_bias)) and one write strength beta = sigmoid(b) per head and token.  q, k and v
     first pass a short causal convolution over time per channel (`taps` wide, last tap on the current token, no bias, continued across

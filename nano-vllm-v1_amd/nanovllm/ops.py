@@ -686,7 +686,7 @@ def attn_paged_any(q, k_cache, v_cache, cu_seqlens_q, context_lens, block_tables
     [pages, G, vdim, page] (transposed within a page, as attn_rotary_prep stores them); out [T, H*vdim].  `slopes` (fp32 [H]):
     score -= slope * distance; `window` > 0: a query sees the last `window` positions and the first `keep_first`; `chunk` > 0: a
     query sees only the keys of its own block of `chunk` positions (counted from the sequence's start); `sinks` (fp32 [H]): a logit
-    per head that joins the softmax's denominator once, with no key and no value."""
+    per head whose exponential is one more term of the softmax's denominator (it stands for no token and carries no value)."""
     f = _act_flag(q, k_cache, v_cache)
     t = q.shape[0]
     batch = context_lens.numel()
